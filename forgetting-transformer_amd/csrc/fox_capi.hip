@@ -1,0 +1,182 @@
+// Flat C ABI of libfox_attn.so: argument validation and kernel dispatch.
+// Declarations and their reference citations live in include/fox_attn.h.
+#include "../../include/fox_attn.h"
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "fox_kernels.hpp"
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+  if (e == hipSuccess) return FOX_OK;
+  return fail(FOX_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+int check_dims(const fox_dims* d) {
+  if (!d) return fail(FOX_E_ARG, "dims is NULL");
+  if (d->B <= 0 || d->H <= 0 || d->M <= 0 || d->N <= 0) return fail(FOX_E_ARG, "B, H, M, N must be positive (got %d, %d, %d, %d)", d->B, d->H, d->M, d->N);
+  if (d->M > d->N) return fail(FOX_E_ARG, "the key/value tensors must be at least as long as the query tensor (M=%d > N=%d)", d->M, d->N);
+  if (d->D != 16 && d->D != 32 && d->D != 64 && d->D != 128) return fail(FOX_E_ARG, "head dim must be one of 16, 32, 64, 128 (got %d)", d->D);
+  if (d->dtype != FOX_DTYPE_BF16 && d->dtype != FOX_DTYPE_FP16) return fail(FOX_E_ARG, "dtype must be FOX_DTYPE_BF16 or FOX_DTYPE_FP16 (got %d)", d->dtype);
+  if ((int64_t)d->B * d->H > 0x7fffffffLL / 4096) return fail(FOX_E_ARG, "B*H too large");
+  return FOX_OK;
+}
+
+int check_view(const fox_view* v, const char* name) {
+  if (!v || !v->ptr) return fail(FOX_E_ARG, "%s is NULL", name);
+  if (((uintptr_t)v->ptr & 15) != 0) return fail(FOX_E_ALIGN, "%s must be 16-byte aligned", name);
+  if ((v->stride_b & 7) || (v->stride_h & 7) || (v->stride_t & 7)) return fail(FOX_E_ALIGN, "strides of %s must be multiples of 8 elements", name);
+  return FOX_OK;
+}
+
+fox::View to_view(const fox_view& v) { return fox::View{(const uint16_t*)v.ptr, v.stride_b, v.stride_h, v.stride_t}; }
+
+#define FOX_TRY(x)            \
+  do {                        \
+    const int rc_ = (x);      \
+    if (rc_ != FOX_OK) return rc_; \
+  } while (0)
+
+int make_bwd(const fox_bwd_args* args, fox::BwdK& k, bool need_grads) {
+  if (!args) return fail(FOX_E_ARG, "args is NULL");
+  FOX_TRY(check_dims(&args->dims));
+  FOX_TRY(check_view(&args->o, "o"));
+  FOX_TRY(check_view(&args->d_o, "do"));
+  if (!args->delta) return fail(FOX_E_ARG, "delta is NULL");
+  k = fox::BwdK{};
+  k.o = to_view(args->o);
+  k.d_o = to_view(args->d_o);
+  k.delta = args->delta;
+  k.B = args->dims.B; k.H = args->dims.H; k.M = args->dims.M; k.N = args->dims.N;
+  k.sm_scale = args->sm_scale;
+  k.n_tiles = 0;
+  if (!need_grads) return FOX_OK;
+  FOX_TRY(check_view(&args->q, "q"));
+  FOX_TRY(check_view(&args->k, "k"));
+  FOX_TRY(check_view(&args->v, "v"));
+  if (!args->log_lambda || !args->lse || !args->dlog_lambda) return fail(FOX_E_ARG, "log_lambda, lse and dlog_lambda must not be NULL");
+  k.q = to_view(args->q);
+  k.k = to_view(args->k);
+  k.v = to_view(args->v);
+  k.c = args->log_lambda;
+  k.lse = args->lse;
+  k.seq_start = args->seq_start;
+  k.thr = args->threshold;
+  k.dc = args->dlog_lambda;
+  return FOX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fox_version(void) { return 100; }  // 0.1.0
+
+const char* fox_last_error(void) { return g_err; }
+
+int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_block_n, int32_t* kv_block_m) {
+  if (D != 16 && D != 32 && D != 64 && D != 128) return fail(FOX_E_ARG, "head dim must be one of 16, 32, 64, 128 (got %d)", D);
+  if (block_m) *block_m = fox::kFwdBM;
+  if (block_n) *block_n = fox::kFwdBN;
+  if (kv_block_n) *kv_block_n = fox::kKvBN;
+  if (kv_block_m) *kv_block_m = fox::kKvBM;
+  return FOX_OK;
+}
+
+int fox_cumsum_fwd(const float* g, int64_t g_sb, int64_t g_sh, int64_t g_sn, const int64_t* seq_start, float* c, int32_t B,
+                   int32_t H, int32_t N, void* stream) {
+  if (!g || !c) return fail(FOX_E_ARG, "g and c must not be NULL");
+  if (B <= 0 || H <= 0 || N <= 0) return fail(FOX_E_ARG, "B, H, N must be positive");
+  return check_hip(fox::launch_cumsum_fwd(g, g_sb, g_sh, g_sn, seq_start, c, B, H, N, (hipStream_t)stream), "fox_cumsum_fwd");
+}
+
+int fox_cumsum_bwd(const float* dc, float* dg, int32_t B, int32_t H, int32_t N, void* stream) {
+  if (!dc || !dg) return fail(FOX_E_ARG, "dc and dg must not be NULL");
+  if (B <= 0 || H <= 0 || N <= 0) return fail(FOX_E_ARG, "B, H, N must be positive");
+  if (dc == dg) return fail(FOX_E_ARG, "dc and dg must not alias");
+  return check_hip(fox::launch_cumsum_bwd(dc, dg, B, H, N, (hipStream_t)stream), "fox_cumsum_bwd");
+}
+
+int fox_auto_threshold(const fox_dims* dims, const fox_view* q, const fox_view* k, float sm_scale, float* thr,
+                       uint32_t* scratch, void* stream) {
+  FOX_TRY(check_dims(dims));
+  FOX_TRY(check_view(q, "q"));
+  FOX_TRY(check_view(k, "k"));
+  if (!thr || !scratch) return fail(FOX_E_ARG, "thr and scratch must not be NULL");
+  return check_hip(fox::launch_auto_threshold(to_view(*q), to_view(*k), dims->B, dims->H, dims->M, dims->N, dims->D,
+                                              dims->dtype, sm_scale, thr, scratch, (hipStream_t)stream),
+                   "fox_auto_threshold");
+}
+
+int fox_attn_fwd(const fox_fwd_args* args, void* stream) {
+  if (!args) return fail(FOX_E_ARG, "args is NULL");
+  FOX_TRY(check_dims(&args->dims));
+  FOX_TRY(check_view(&args->q, "q"));
+  FOX_TRY(check_view(&args->k, "k"));
+  FOX_TRY(check_view(&args->v, "v"));
+  FOX_TRY(check_view(&args->o, "o"));
+  if (!args->log_lambda || !args->lse) return fail(FOX_E_ARG, "log_lambda and lse must not be NULL");
+  fox::FwdK k{};
+  k.q = to_view(args->q);
+  k.k = to_view(args->k);
+  k.v = to_view(args->v);
+  k.o = to_view(args->o);
+  k.c = args->log_lambda;
+  k.lse = args->lse;
+  k.seq_start = args->seq_start;
+  k.thr = args->threshold;
+  k.first_block = args->first_block;
+  k.B = args->dims.B; k.H = args->dims.H; k.M = args->dims.M; k.N = args->dims.N;
+  k.sm_scale = args->sm_scale;
+  k.n_mtiles = (args->dims.M + fox::kFwdBM - 1) / fox::kFwdBM;
+  return check_hip(fox::launch_fwd(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), "fox_attn_fwd");
+}
+
+int fox_attn_bwd_delta(const fox_bwd_args* args, void* stream) {
+  fox::BwdK k;
+  FOX_TRY(make_bwd(args, k, false));
+  return check_hip(fox::launch_bwd_delta(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), "fox_attn_bwd_delta");
+}
+
+int fox_attn_bwd_dkdv(const fox_bwd_args* args, void* stream) {
+  fox::BwdK k;
+  FOX_TRY(make_bwd(args, k, true));
+  FOX_TRY(check_view(&args->dk, "dk"));
+  FOX_TRY(check_view(&args->dv, "dv"));
+  k.dk = to_view(args->dk);
+  k.dv = to_view(args->dv);
+  return check_hip(fox::launch_bwd_dkdv(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), "fox_attn_bwd_dkdv");
+}
+
+int fox_attn_bwd_dq(const fox_bwd_args* args, void* stream) {
+  fox::BwdK k;
+  FOX_TRY(make_bwd(args, k, true));
+  FOX_TRY(check_view(&args->dq, "dq"));
+  k.dq = to_view(args->dq);
+  return check_hip(fox::launch_bwd_dq(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), "fox_attn_bwd_dq");
+}
+
+int fox_attn_bwd(const fox_bwd_args* args, void* stream) {
+  if (!args) return fail(FOX_E_ARG, "args is NULL");
+  if (!args->dlog_fgate) return fail(FOX_E_ARG, "dlog_fgate is NULL");
+  FOX_TRY(fox_attn_bwd_delta(args, stream));
+  FOX_TRY(fox_attn_bwd_dkdv(args, stream));
+  FOX_TRY(fox_attn_bwd_dq(args, stream));
+  return fox_cumsum_bwd(args->dlog_lambda, args->dlog_fgate, args->dims.B, args->dims.H, args->dims.N, stream);
+}
+
+}  // extern "C"

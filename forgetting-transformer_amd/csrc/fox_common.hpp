@@ -1,0 +1,231 @@
+// Shared device-side building blocks for the gfx950 Forgetting Attention kernels:
+// vector types, MFMA wrappers, the swizzled LDS tile layout with its two read
+// patterns (row operand via ds_read_b128, transposed operand via
+// ds_read_b64_tr_b16), the global->LDS tile loader and small wave helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fox {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------------------
+// Element traits: bf16 and fp16 share every kernel; only the MFMA opcode and the
+// fp32 <-> 16-bit conversions differ.
+// ---------------------------------------------------------------------------
+struct Bf16 {
+  static __device__ inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ inline uint32_t pack2(float lo, float hi) {
+    bf16x2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ inline float lo(uint32_t w) { return __uint_as_float(w << 16); }
+  static __device__ inline float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+};
+
+struct Fp16 {
+  static __device__ inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ inline uint32_t pack2(float lo, float hi) {
+    f16x2 v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ inline float lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
+  static __device__ inline float hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
+};
+
+// Pack eight consecutive accumulator values into one 16-byte MFMA operand.
+template <typename Tr>
+__device__ inline u32x4 pack8(const f32x16& c, int first) {
+  u32x4 r;
+  r[0] = Tr::pack2(c[first + 0], c[first + 1]);
+  r[1] = Tr::pack2(c[first + 2], c[first + 3]);
+  r[2] = Tr::pack2(c[first + 4], c[first + 5]);
+  r[3] = Tr::pack2(c[first + 6], c[first + 7]);
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// MFMA 32x32x16 register layouts (lane = 32*g + i):
+//   A operand: row i,  k = 8*g .. 8*g+7          B operand: col i, same k
+//   C/D:       col i,  row(r) = 8*(r/4) + 4*g + r%4   for r = 0..15
+// A C tile can feed the next MFMA as its B operand with the C rows as the
+// contraction index: operand element e = 4*u + t of k-slice h (16 rows) is
+// accumulator register r = 8*h + e, i.e. C row 16*h + 8*u + 4*g + t.
+// ---------------------------------------------------------------------------
+__device__ inline int c_row(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+
+// ---------------------------------------------------------------------------
+// LDS tile: ROWS x D 16-bit elements, dense rows of D*2 bytes, 16-byte chunks
+// XOR-swizzled by a row-dependent pattern so that both read patterns below
+// spread over all banks.
+// ---------------------------------------------------------------------------
+template <int D>
+struct Tile {
+  static constexpr int CH = D / 8;
+  static constexpr int ROW_BYTES = D * 2;
+  static __device__ inline int swz(int row) {
+    if constexpr (CH == 16) return ((row & 3) << 2) | ((row >> 2) & 3);
+    else if constexpr (CH == 8) return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+    else if constexpr (CH == 4) return (row >> 2) & 3;
+    else return (row >> 3) & 1;
+  }
+  static __device__ inline int off(int row, int chunk) { return row * ROW_BYTES + ((chunk ^ swz(row)) << 4); }
+};
+
+// Row operand: eight consecutive elements (one chunk) of one row.
+template <int D>
+__device__ inline u32x4 lds_row_operand(const char* tile, int row, int chunk) {
+  return *reinterpret_cast<const u32x4*>(tile + Tile<D>::off(row, chunk));
+}
+
+__device__ inline u32x2 lds_tr_read(const char* p) {
+  typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+  return __builtin_bit_cast(u32x2, v);
+}
+
+// Transposed operand for k-slice rows [row16, row16+16) and the 32 columns
+// [32*db, 32*db+32): lane (g, i) receives column 32*db + i at rows
+// row16 + 8*u + 4*g + t (element 4*u + t).  ds_read_b64_tr_b16 works on blocks of
+// 16 lanes: lane x of a block supplies the address of 4 consecutive columns
+// 4*(x%4).. of row (x/4), and receives column x of those four rows.
+template <int D>
+__device__ inline u32x4 lds_col_operand(const char* tile, int row16, int db, int lane) {
+  const int g = lane >> 5, blk = (lane >> 4) & 1, x = lane & 15;
+  int col = 32 * db + 16 * blk + 4 * (x & 3);
+  if constexpr (D < 32) col &= (D - 1);  // columns >= D feed output rows nobody stores
+  const int row = row16 + 4 * g + (x >> 2);
+  const int inner = (col & 7) * 2;
+  u32x2 lo = lds_tr_read(tile + Tile<D>::off(row, col >> 3) + inner);
+  u32x2 hi = lds_tr_read(tile + Tile<D>::off(row + 8, col >> 3) + inner);
+  u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// Global -> register -> LDS loader for a ROWS x D tile of 16-bit elements.
+// Rows at or beyond row_limit read as zero.  Split into load() and store() so the
+// global loads of the next tile fly while the current one is consumed.
+// ---------------------------------------------------------------------------
+template <int D, int ROWS, int NT>
+struct TileLoader {
+  static constexpr int CH = D / 8;
+  static constexpr int CHUNKS = ROWS * CH;
+  static constexpr int PER = (CHUNKS + NT - 1) / NT;
+  u32x4 reg[PER];
+
+  __device__ inline void load(const uint16_t* base, int64_t row_stride, int row0, int row_limit, int tid) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int idx = tid + j * NT;
+      const int row = idx / CH, ch = idx % CH;
+      u32x4 z = {0u, 0u, 0u, 0u};
+      reg[j] = z;
+      if ((CHUNKS % NT == 0 || idx < CHUNKS) && row0 + row < row_limit)
+        reg[j] = *reinterpret_cast<const u32x4*>(base + (int64_t)(row0 + row) * row_stride + ch * 8);
+    }
+  }
+  __device__ inline void store(char* tile, int tid) const {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int idx = tid + j * NT;
+      const int row = idx / CH, ch = idx % CH;
+      if (CHUNKS % NT == 0 || idx < CHUNKS) *reinterpret_cast<u32x4*>(tile + Tile<D>::off(row, ch)) = reg[j];
+    }
+  }
+};
+
+// Operand held in registers for a whole kernel: lane (g, i) keeps row (row0 + i),
+// elements 16*kk + 8*g .. +7 for every k-step kk.  Rows >= row_limit are zero.
+template <int D>
+__device__ inline void load_row_operand_regs(u32x4 (&dst)[D / 16], const uint16_t* base, int64_t row_stride, int row,
+                                             int row_limit, int g) {
+#pragma unroll
+  for (int kk = 0; kk < D / 16; ++kk) {
+    u32x4 z = {0u, 0u, 0u, 0u};
+    dst[kk] = z;
+    if (row < row_limit) dst[kk] = *reinterpret_cast<const u32x4*>(base + (int64_t)row * row_stride + 16 * kk + 8 * g);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Wave helpers
+// ---------------------------------------------------------------------------
+// Value held by the partner lane in the other 32-lane half.
+__device__ inline float half_max(float x) {
+  unsigned v = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ inline float half_sum(float x) {
+  unsigned v = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// Workgroup id -> (bh, tile) with every tile of one (batch, head) on one XCD (the
+// hardware deals consecutive workgroup ids round-robin over 8 XCDs, each with its
+// own L2), heaviest tiles (largest index under a causal mask) first.
+__device__ inline void decode_block(int wid, int n_tiles, int n_bh, int& bh, int& tile) {
+  if ((n_bh & 7) == 0) {
+    const int xcd = wid & 7, seq = wid >> 3;
+    bh = (seq / n_tiles) * 8 + xcd;
+    tile = n_tiles - 1 - (seq % n_tiles);
+  } else {
+    bh = wid / n_tiles;
+    tile = n_tiles - 1 - (wid % n_tiles);
+  }
+}
+
+// Adaptive Computation Pruning, query-side bound: the first key block of width BN
+// in [0, t_max] whose largest decay  c_out - c[last column of the block]  is not
+// below thr.  c is non-increasing, so the blocks before it are exactly the
+// prunable ones.  Evaluated by all 64 lanes at once; the result is wave-uniform.
+__device__ inline int acp_first_kept_block(const float* c_row, float c_out, float thr, int N, int BN, int t_max, int lane) {
+  for (int base = 0; base <= t_max; base += kWave) {
+    const int t = base + lane;
+    bool keep = false;
+    if (t <= t_max) {
+      int col = t * BN + BN - 1;
+      col = col < N - 1 ? col : N - 1;
+      keep = !((c_out - c_row[col]) < thr);
+    }
+    const unsigned long long m = __ballot(keep);
+    if (m) return base + __ffsll((long long)m) - 1;
+  }
+  return t_max;
+}
+
+// Key-side bound: the first query block (BMQ rows, first row u*BMQ) in [u_lo, U)
+// whose largest decay against the key tile,  c[P_SEQ + u*BMQ] - c_last,  is below
+// thr; every later block is prunable too.  Returns U when none is.
+__device__ inline int acp_first_pruned_qblock(const float* c_row, float c_last, float thr, int p_seq, int BMQ, int u_lo,
+                                              int U, int lane) {
+  for (int base = u_lo; base < U; base += kWave) {
+    const int u = base + lane;
+    bool pruned = false;
+    if (u < U) pruned = (c_row[p_seq + u * BMQ] - c_last) < thr;
+    const unsigned long long m = __ballot(pruned);
+    if (m) return base + __ffsll((long long)m) - 1;
+  }
+  return U;
+}
+
+}  // namespace fox

@@ -1,0 +1,55 @@
+// Kernel argument blocks and launcher declarations shared by the C ABI layer and
+// the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fox {
+
+struct View {
+  const uint16_t* ptr;
+  int64_t sb, sh, st;
+};
+
+struct FwdK {
+  View q, k, v, o;
+  const float* c;
+  float* lse;
+  const int64_t* seq_start;
+  const float* thr;
+  int32_t* first_block;
+  int B, H, M, N;
+  float sm_scale;
+  int n_mtiles;
+};
+
+struct BwdK {
+  View q, k, v, o, d_o, dq, dk, dv;
+  const float* c;
+  const float* lse;
+  const int64_t* seq_start;
+  const float* thr;
+  float* delta;
+  float* dc;
+  int B, H, M, N;
+  float sm_scale;
+  int n_tiles;
+};
+
+// Tile sizes (see fox_tile_config in the public header)
+constexpr int kFwdBM = 128;
+constexpr int kFwdBN = 64;
+constexpr int kKvBN = 128;   // key rows per workgroup in the dK/dV kernel
+constexpr int kKvBM = 32;    // query rows per step in the dK/dV kernel
+
+hipError_t launch_fwd(const FwdK& a, int D, int dtype, hipStream_t s);
+hipError_t launch_bwd_delta(const BwdK& a, int D, int dtype, hipStream_t s);
+hipError_t launch_bwd_dkdv(const BwdK& a, int D, int dtype, hipStream_t s);
+hipError_t launch_bwd_dq(const BwdK& a, int D, int dtype, hipStream_t s);
+hipError_t launch_cumsum_fwd(const float* g, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start, float* c, int B,
+                             int H, int N, hipStream_t s);
+hipError_t launch_cumsum_bwd(const float* dc, float* dg, int B, int H, int N, hipStream_t s);
+hipError_t launch_auto_threshold(const View& q, const View& k, int B, int H, int M, int N, int D, int dtype, float sm_scale,
+                                 float* thr, uint32_t* scratch, hipStream_t s);
+
+}  // namespace fox

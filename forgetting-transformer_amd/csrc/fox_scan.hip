@@ -1,0 +1,164 @@
+// Row scans and the "auto" pruning threshold for gfx950.
+//
+//   scan_kernel<false> : c[n]  = sum_{l<=n} g[l], with g[l] := 0 for l < seq_start
+//   scan_kernel<true>  : dg[l] = sum_{n>=l} dc[n]
+//   norm_max_kernel / threshold_kernel : the "auto" threshold from the largest row
+//                        L2 norms of q and k.
+//
+// One workgroup scans one (batch, head) row.  Partial sums are carried in fp64 and
+// rounded once on store, so c is exactly non-increasing whenever g <= 0 (the
+// pruning bounds rely on that) and long rows lose no precision to the scan order.
+#include "fox_common.hpp"
+#include "fox_kernels.hpp"
+
+namespace fox {
+
+template <bool REVERSE>
+__global__ __launch_bounds__(256) void scan_kernel(const float* __restrict__ in, int64_t sb, int64_t sh, int64_t sn,
+                                                   const int64_t* __restrict__ seq_start, float* __restrict__ out, int H,
+                                                   int N) {
+  constexpr int PER = 4, NT = 256, SPAN = PER * NT;
+  __shared__ double wave_tot[NT / kWave];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.x, b = bh / H, h = bh % H;
+  const float* src = in + b * sb + h * sh;
+  float* dst = out + (int64_t)bh * N;
+  int seq = 0;
+  if (!REVERSE && seq_start) {
+    const int64_t s64 = seq_start[b];
+    seq = (int)(s64 < 0 ? 0 : (s64 > N ? N : s64));
+  }
+  double carry = 0.0;
+  for (int base = 0; base < N; base += SPAN) {
+    double v[PER];
+    double run = 0.0;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const int pos = base + tid * PER + e;            // position in scan order
+      const int idx = REVERSE ? N - 1 - pos : pos;     // element index
+      float x = 0.f;
+      if (pos < N && (REVERSE || idx >= seq)) x = src[(int64_t)idx * sn];
+      run += (double)x;
+      v[e] = run;
+    }
+    // inclusive scan of the per-thread totals across the wave, then across waves
+    double incl = run;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const double up = __shfl_up(incl, off);
+      if (lane >= off) incl += up;
+    }
+    if (lane == kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    double before = carry, total = 0.0;
+#pragma unroll
+    for (int w = 0; w < NT / kWave; ++w) {
+      const double t = wave_tot[w];
+      if (w < wave) before += t;
+      total += t;
+    }
+    before += incl - run;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const int pos = base + tid * PER + e;
+      const int idx = REVERSE ? N - 1 - pos : pos;
+      if (pos < N) dst[idx] = (float)(before + v[e]);
+    }
+    carry += total;
+    __syncthreads();
+  }
+}
+
+hipError_t launch_cumsum_fwd(const float* g, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start, float* c, int B,
+                             int H, int N, hipStream_t s) {
+  hipLaunchKernelGGL(scan_kernel<false>, dim3((unsigned)(B * H)), dim3(256), 0, s, g, sb, sh, sn, seq_start, c, H, N);
+  return hipGetLastError();
+}
+
+hipError_t launch_cumsum_bwd(const float* dc, float* dg, int B, int H, int N, hipStream_t s) {
+  hipLaunchKernelGGL(scan_kernel<true>, dim3((unsigned)(B * H)), dim3(256), 0, s, dc, (int64_t)H * N, (int64_t)N, (int64_t)1,
+                     (const int64_t*)nullptr, dg, H, N);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// "auto" threshold
+// ---------------------------------------------------------------------------
+template <typename Tr>
+__device__ inline float round16(float x) {  // round to the 16-bit dtype and back
+  return Tr::lo(Tr::pack2(x, 0.f));
+}
+
+__global__ void zero_u32_kernel(uint32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// grid (row blocks, B*H, 2): z = 0 scans q (T = M), z = 1 scans k (T = N).
+template <typename Tr, int D>
+__global__ __launch_bounds__(256) void norm_max_kernel(View q, View k, int H, int M, int N, uint32_t* scratch) {
+  constexpr int LPR = D / 8, RPP = 256 / LPR, ROWS = 512;
+  const int tid = threadIdx.x;
+  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  const View& t = blockIdx.z == 0 ? q : k;
+  const int T = blockIdx.z == 0 ? M : N;
+  const uint16_t* p = t.ptr + b * t.sb + h * t.sh;
+  const int ch = tid % LPR;
+  float best = 0.f;
+  for (int pass = 0; pass < ROWS / RPP; ++pass) {
+    const int row = blockIdx.x * ROWS + pass * RPP + tid / LPR;
+    float acc = 0.f;
+    if (row < T) {
+      const u32x4 x = *reinterpret_cast<const u32x4*>(p + (int64_t)row * t.st + ch * 8);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc += Tr::lo(x[e]) * Tr::lo(x[e]) + Tr::hi(x[e]) * Tr::hi(x[e]);
+    }
+#pragma unroll
+    for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+    best = fmaxf(best, round16<Tr>(sqrtf(acc)));
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) best = fmaxf(best, __shfl_xor(best, off));
+  if ((tid & 63) == 0) atomicMax(&scratch[bh * 2 + blockIdx.z], __float_as_uint(best));  // non-negative floats order like uints
+}
+
+template <typename Tr>
+__global__ void threshold_kernel(const uint32_t* scratch, float* thr, int n_bh, float sm_scale, float log_n) {
+  const int bh = blockIdx.x * blockDim.x + threadIdx.x;
+  if (bh >= n_bh) return;
+  const float qn = __uint_as_float(scratch[bh * 2]), kn = __uint_as_float(scratch[bh * 2 + 1]);
+  // every tensor op of the reference rounds to the input dtype
+  float ub = round16<Tr>(qn * kn);
+  ub = round16<Tr>(ub * sm_scale);
+  float t = round16<Tr>(2.f * ub);
+  t = round16<Tr>(t + log_n);
+  t = -t;
+  t = round16<Tr>(t - 10.f);
+  thr[bh] = t;
+}
+
+template <typename Tr>
+static hipError_t auto_threshold_t(const View& q, const View& k, int B, int H, int M, int N, int D, float sm_scale, float* thr,
+                                   uint32_t* scratch, hipStream_t s) {
+  const int n_bh = B * H;
+  hipLaunchKernelGGL(zero_u32_kernel, dim3((unsigned)((2 * n_bh + 255) / 256)), dim3(256), 0, s, scratch, 2 * n_bh);
+  const dim3 grid((unsigned)((N + 511) / 512), (unsigned)n_bh, 2u);
+  switch (D) {
+    case 16: hipLaunchKernelGGL((norm_max_kernel<Tr, 16>), grid, dim3(256), 0, s, q, k, H, M, N, scratch); break;
+    case 32: hipLaunchKernelGGL((norm_max_kernel<Tr, 32>), grid, dim3(256), 0, s, q, k, H, M, N, scratch); break;
+    case 64: hipLaunchKernelGGL((norm_max_kernel<Tr, 64>), grid, dim3(256), 0, s, q, k, H, M, N, scratch); break;
+    case 128: hipLaunchKernelGGL((norm_max_kernel<Tr, 128>), grid, dim3(256), 0, s, q, k, H, M, N, scratch); break;
+    default: return hipErrorInvalidValue;
+  }
+  hipLaunchKernelGGL((threshold_kernel<Tr>), dim3((unsigned)((n_bh + 255) / 256)), dim3(256), 0, s, scratch, thr, n_bh,
+                     sm_scale, (float)log((double)N));
+  return hipGetLastError();
+}
+
+hipError_t launch_auto_threshold(const View& q, const View& k, int B, int H, int M, int N, int D, int dtype, float sm_scale,
+                                 float* thr, uint32_t* scratch, hipStream_t s) {
+  return dtype == 0 ? auto_threshold_t<Bf16>(q, k, B, H, M, N, D, sm_scale, thr, scratch, s)
+                    : auto_threshold_t<Fp16>(q, k, B, H, M, N, D, sm_scale, thr, scratch, s);
+}
+
+}  // namespace fox

@@ -1,0 +1,11 @@
+"""Forgetting Attention for AMD MI355X (gfx950).
+
+Same import path and call signature as the reference package
+(``src/forgetting_transformer/__init__.py:1-3``)::
+
+    from forgetting_transformer import forgetting_attention
+"""
+from .ops.forgetting_attention import forgetting_attention
+
+__version__ = "0.1.0"
+__all__ = ["forgetting_attention"]

@@ -1,0 +1,236 @@
+"""Forgetting Attention on AMD MI355X: host side of the operator.
+
+This module mirrors the public surface of the reference's
+``src/forgetting_transformer/ops/forgetting_attention.py`` -- the function
+``forgetting_attention`` (``:403-455``) and the ``torch.autograd.Function``
+``ForgettingAttention`` (``:44-400``) with the same argument order, checks and
+error types -- but every device computation is done by hand-written gfx950 HIP
+kernels reached through the flat C ABI of ``libfox_attn.so``.  PyTorch only
+provides device memory, the current stream and autograd bookkeeping.  There is no
+fallback path: without the library, or with tensors that are not on a GPU, the
+call raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Literal, Optional, Union
+
+import torch
+
+from . import _lib
+
+__all__ = ["forgetting_attention", "ForgettingAttention"]
+
+_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
+
+
+def maybe_contiguous(x: torch.Tensor) -> torch.Tensor:
+    """Make ``x`` usable by the kernels without copying when possible.
+
+    The reference only requires a unit innermost stride (``:35-38``); the HIP
+    kernels read 16-byte vectors, so the base pointer must also be 16-byte aligned
+    and the outer strides multiples of 8 elements.  Anything else is copied.
+    """
+    ok = x.stride(-1) == 1 and x.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in x.stride()[:-1])
+    return x if ok else x.contiguous()
+
+
+def _view(x: torch.Tensor) -> _lib.View:
+    return _lib.View(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2))
+
+
+def _ptr(x: Optional[torch.Tensor]):
+    return None if x is None else C.c_void_p(x.data_ptr())
+
+
+def _stream(device: torch.device):
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+class ForgettingAttention(torch.autograd.Function):
+    """Autograd node; argument list identical to the reference's (``:72-73``).
+
+    ``record_time_key`` / ``record_attention_time`` / ``record_find_index_time``
+    (the reference's in-op CUDA-event timers, ``:45-70``) are accepted for
+    signature compatibility but must be off: kernels here are timed from outside
+    with a profiler.
+    """
+
+    @staticmethod
+    def forward(ctx, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
+                return_log_normalizer=False, return_start_index=False, record_time_key=None,
+                record_attention_time=False, record_find_index_time=False):
+        assert causal, "Only causal attention is supported"
+        assert not (record_attention_time or record_find_index_time), \
+            "in-op timers are not implemented; profile the kernels with rocprofv3 instead"
+        Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
+        assert Dq == Dk == Dv, "feature size of q, k, v should be equal"
+        assert Dk in {16, 32, 64, 128}, "We only support head dims in {16, 32, 64, 128}"
+        assert q.dtype == k.dtype == v.dtype, "q, k, v must share one dtype"
+
+        B, H, M, D = q.shape
+        N = k.shape[2]
+        assert log_fgate.shape == (B, H, N)
+        assert log_fgate.dtype == torch.float32, (
+            "log_fgate must be in torch.float32. It is best to do this cast before logsigmoid, "
+            "e.g., torch.nn.functional.logsigmoid(fgate_logit.float()).")
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(D)
+        sm_scale = float(sm_scale)
+
+        Hk, Hv = k.shape[1], v.shape[1]
+        assert Hk == Hv, "num of heads in k and v should be equal"
+        assert H == Hk, "groupped query attention has not been tested. You can uncomment this if you know what you are doing."
+        assert k.shape == (B, Hk, N, D) and v.shape == (B, Hv, N, D)
+        assert not (M > N), "The key/value tensors must be longer than the query tensor"
+
+        # threshold: validate on the host first (:91-109), compute "auto" on the device later
+        auto_threshold = False
+        if adaptive_threshold is not None:
+            if isinstance(adaptive_threshold, str):
+                assert adaptive_threshold == "auto", (
+                    'adaptive_threshold must be either the string "auto", a float, or a Tensor, '
+                    f"but got {adaptive_threshold}.")
+                auto_threshold = True
+            else:
+                adaptive_threshold = torch.as_tensor(adaptive_threshold, dtype=torch.float, device=q.device)
+                try:
+                    adaptive_threshold = torch.broadcast_to(adaptive_threshold, (B, H))
+                except RuntimeError:
+                    raise RuntimeError(
+                        'adaptive_threshold must be either the string "auto" or broadcastable to '
+                        f"(batch_size, num_heads) = ({B}, {H}), but got {adaptive_threshold.size()}.")
+                assert adaptive_threshold.size() == (B, H)
+                adaptive_threshold = adaptive_threshold.contiguous()
+
+        if seq_start is not None:
+            has_seq_start = True
+            assert seq_start.shape == (B,)
+        else:
+            has_seq_start = False
+
+        if q.device.type != "cuda":
+            raise RuntimeError("forgetting_attention runs only on an AMD GPU (HIP device); "
+                               f"got tensors on '{q.device}'. There is no CPU implementation.")
+        lib = _lib.load()
+        device = q.device
+        dims = _lib.Dims(B, H, M, N, D, _DTYPES[q.dtype])
+        if has_seq_start:
+            seq_start = seq_start.to(device=device, dtype=torch.long).contiguous()
+
+        q, k, v = maybe_contiguous(q), maybe_contiguous(k), maybe_contiguous(v)
+
+        with torch.cuda.device(device):
+            stream = _stream(device)
+
+            if auto_threshold:
+                adaptive_threshold = torch.empty((B, H), dtype=torch.float32, device=device)
+                scratch = torch.empty((B, H, 2), dtype=torch.int32, device=device)
+                qv, kv = _view(q), _view(k)
+                _lib.check(lib.fox_auto_threshold(C.byref(dims), C.byref(qv), C.byref(kv), sm_scale,
+                                                  _ptr(adaptive_threshold), _ptr(scratch), stream), "fox_auto_threshold")
+
+            # c = cumsum(log_fgate) with gates left of seq_start zeroed, one fused kernel
+            log_lambda = torch.empty((B, H, N), dtype=torch.float32, device=device)
+            _lib.check(lib.fox_cumsum_fwd(_ptr(log_fgate), log_fgate.stride(0), log_fgate.stride(1), log_fgate.stride(2),
+                                          _ptr(seq_start), _ptr(log_lambda), B, H, N, stream), "fox_cumsum_fwd")
+
+            o = torch.empty_like(q)
+            L = torch.empty((B, H, M), device=device, dtype=torch.float32)
+            first_block = None
+            if return_start_index:
+                block_m, _, _, _ = _lib.tile_config(D)
+                first_block = torch.zeros((B, H, (M + block_m - 1) // block_m), dtype=torch.int32, device=device)
+            args = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), log_lambda.data_ptr(), L.data_ptr(),
+                                None if seq_start is None else seq_start.data_ptr(),
+                                None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
+                                sm_scale, None if first_block is None else first_block.data_ptr())
+            _lib.check(lib.fox_attn_fwd(C.byref(args), stream), "fox_attn_fwd")
+
+        ctx.save_for_backward(q, k, v, o, L, log_lambda, seq_start, adaptive_threshold)
+        ctx.sm_scale = sm_scale
+        ctx.causal = causal
+        ctx.has_seq_start = has_seq_start
+
+        if return_log_normalizer or return_start_index:
+            start_index = None
+            if return_start_index:
+                _, block_n, _, _ = _lib.tile_config(D)
+                start_index = first_block.to(torch.long) * block_n
+            outs = (o, L if return_log_normalizer else None, start_index)
+            ctx.mark_non_differentiable(*[t for t in outs[1:] if t is not None])
+            return outs
+        return o
+
+    @staticmethod
+    def backward(ctx, do, *ignored):
+        q, k, v, o, L, log_lambda, seq_start, adaptive_threshold = ctx.saved_tensors
+        B, H, M, D = q.shape
+        N = k.shape[2]
+        device = q.device
+        lib = _lib.load()
+        do = maybe_contiguous(do)
+        with torch.cuda.device(device):
+            stream = _stream(device)
+            delta = torch.empty_like(L)
+            dlog_lambda = torch.empty((B, H, N), dtype=torch.float32, device=device)
+            dlog_fgate = torch.empty((B, H, N), dtype=torch.float32, device=device)
+            dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+            args = _lib.BwdArgs(
+                _lib.Dims(B, H, M, N, D, _DTYPES[q.dtype]),
+                _view(q), _view(k), _view(v), _view(o), _view(do), _view(dq), _view(dk), _view(dv),
+                log_lambda.data_ptr(), L.data_ptr(),
+                None if seq_start is None else seq_start.data_ptr(),
+                None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
+                ctx.sm_scale, delta.data_ptr(), dlog_lambda.data_ptr(), dlog_fgate.data_ptr())
+            _lib.check(lib.fox_attn_bwd(C.byref(args), stream), "fox_attn_bwd")
+        return dq, dk, dv, dlog_fgate, None, None, None, None, None, None, None, None, None
+
+
+def forgetting_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    log_fgate: torch.Tensor,
+    *,
+    head_first: bool = False,
+    seq_start: Optional[torch.Tensor] = None,
+    sm_scale: Optional[float] = None,
+    adaptive_threshold: Optional[Union[Literal["auto"], float, torch.Tensor]] = None,
+):
+    """Causal softmax attention with a data-dependent forget-gate decay bias.
+
+    Same contract as the reference (``:403-455``):
+
+    - q, k, v are bfloat16/float16, log_fgate is float32
+    - seqlen_q <= seqlen_k; query ``i`` sits at key position ``i + seqlen_k - seqlen_q``
+    - head dim in {16, 32, 64, 128}
+
+    Arguments:
+        q: (batch, seqlen_q, heads, head_dim) unless head_first=True.
+        k, v: (batch, seqlen_k, heads, head_dim) unless head_first=True.
+        log_fgate: (batch, seqlen_k, heads) unless head_first=True; the log of the
+            forget gates, typically ``logsigmoid(logits.float())``.
+        head_first: heads axis before the sequence axis in all inputs and the output.
+        seq_start: optional LongTensor (batch,); keys before ``seq_start[b]`` get no
+            attention (left padding).
+        sm_scale: score scale, default ``1/sqrt(head_dim)``.
+        adaptive_threshold: Adaptive Computation Pruning threshold: ``"auto"``, a
+            float, or a tensor broadcastable to (batch, heads).  Key blocks whose
+            decay bias is below it for a whole query block are skipped.
+
+    Returns:
+        out: same shape, layout and dtype as q.
+    """
+    for name, entry in dict(q=q, k=k, v=v).items():
+        assert entry.dtype in [torch.float16, torch.bfloat16], (
+            f"Only torch.float16 or torch.bfloat16 are supported for q/k/v, but got {entry.dtype} for {name}.")
+    if not head_first:
+        q, k, v = [item.transpose(1, 2) for item in (q, k, v)]  # b t h d -> b h t d, views
+        log_fgate = log_fgate.transpose(1, 2)                   # b t h -> b h t
+    out = ForgettingAttention.apply(q, k, v, log_fgate, seq_start, True, sm_scale, adaptive_threshold,
+                                    False, False, None, False, False)
+    if not head_first:
+        out = out.transpose(1, 2)
+    return out

@@ -1,0 +1,130 @@
+/*
+ * fox_attn.h -- flat C ABI of libfox_attn.so: Forgetting Attention for AMD gfx950.
+ *
+ * Every function takes raw device pointers, element strides and a HIP stream
+ * (passed as void*), launches on that stream without synchronising, allocates
+ * nothing and returns 0 on success or a negative FOX_E_* code; fox_last_error()
+ * gives the message of the calling thread's last failure.  The caller owns all
+ * buffers.  Citations name the interface of the reference implementation
+ * (src/forgetting_transformer/ops/forgetting_attention.py) that each entry point
+ * replaces.
+ *
+ * Tensors q, k, v, o, do, dq, dk, dv are 16-bit (bf16 or fp16) with logical shape
+ * (B, H, T, D), arbitrary element strides for B, H, T, unit stride for D; base
+ * pointers must be 16-byte aligned and strides multiples of 8 elements.
+ * D is one of 16, 32, 64, 128.  M = query length, N = key length, M <= N; query
+ * row i sits at key position i + (N - M).
+ */
+#ifndef FOX_ATTN_H
+#define FOX_ATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FOX_OK 0
+#define FOX_E_ARG (-1)     /* null pointer, bad size, unsupported head dim / dtype */
+#define FOX_E_ALIGN (-2)   /* pointer or stride alignment */
+#define FOX_E_LAUNCH (-3)  /* HIP reported a launch failure */
+
+#define FOX_DTYPE_BF16 0
+#define FOX_DTYPE_FP16 1
+
+/* A (B, H, T, D) tensor view: element strides of the first three axes. */
+typedef struct fox_view {
+  void* ptr;
+  int64_t stride_b, stride_h, stride_t;
+} fox_view;
+
+typedef struct fox_dims {
+  int32_t B, H, M, N, D;
+  int32_t dtype; /* FOX_DTYPE_* */
+} fox_dims;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int fox_version(void);
+const char* fox_last_error(void);
+
+/*
+ * Tile sizes the kernels use for a head dim: block_m/block_n of the forward and
+ * dQ kernels (pruning bounds are multiples of block_n per block_m query rows),
+ * and kv_block_n/kv_block_m of the dK/dV kernel.
+ * Replaces get_fwd_config / get_bwd_kv_config / get_bwd_q_config (:460-493, :838-890).
+ */
+int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_block_n, int32_t* kv_block_m);
+
+/*
+ * c[b,h,n] = sum_{l<=n} g[b,h,l] with g[b,h,l] taken as 0 for l < seq_start[b].
+ * g is fp32 with element strides (g_sb, g_sh, g_sn); c is (B,H,N) contiguous fp32.
+ * seq_start may be NULL.  Replaces the prologue at :117-127 (clone, masked zero
+ * fill, torch.cumsum).
+ */
+int fox_cumsum_fwd(const float* g, int64_t g_sb, int64_t g_sh, int64_t g_sn, const int64_t* seq_start, float* c,
+                   int32_t B, int32_t H, int32_t N, void* stream);
+
+/*
+ * dg[b,h,l] = sum_{n>=l} dc[b,h,n]; both (B,H,N) contiguous fp32.
+ * Replaces the reverse cumulative sum at :390-392.
+ */
+int fox_cumsum_bwd(const float* dc, float* dg, int32_t B, int32_t H, int32_t N, void* stream);
+
+/*
+ * thr[b,h] = -(2 * max_m|q| * max_n|k| * sm_scale + log N) - 10, with the row norms
+ * and every intermediate rounded to the input dtype as the reference's tensor
+ * arithmetic does (:95-102).  thr is (B,H) contiguous fp32; scratch is 2*B*H
+ * uint32 that this call overwrites.
+ */
+int fox_auto_threshold(const fox_dims* dims, const fox_view* q, const fox_view* k, float sm_scale, float* thr,
+                       uint32_t* scratch, void* stream);
+
+typedef struct fox_fwd_args {
+  fox_dims dims;
+  fox_view q, k, v, o;        /* o is written */
+  const float* log_lambda;    /* (B,H,N) contiguous, from fox_cumsum_fwd */
+  float* lse;                 /* (B,H,M) contiguous, written: log of the softmax normaliser, -inf for empty rows */
+  const int64_t* seq_start;   /* (B,) or NULL */
+  const float* threshold;     /* (B,H) contiguous or NULL (no pruning) */
+  float sm_scale;
+  int32_t* first_block;       /* optional (B,H,ceil(M/block_m)): first key block each query block visits */
+} fox_fwd_args;
+
+/*
+ * Forward: o = softmax(q k^T sm_scale + c_i - c_j over seq_start <= j <= i+N-M) v.
+ * Replaces _find_start_index_kernel (:695-745) + _fwd_kernel (:505-693) as launched
+ * by ForgettingAttention.forward (:159-204).
+ */
+int fox_attn_fwd(const fox_fwd_args* args, void* stream);
+
+typedef struct fox_bwd_args {
+  fox_dims dims;
+  fox_view q, k, v, o, d_o;   /* inputs */
+  fox_view dq, dk, dv;        /* written */
+  const float* log_lambda;    /* (B,H,N) */
+  const float* lse;           /* (B,H,M) from the forward */
+  const int64_t* seq_start;   /* (B,) or NULL */
+  const float* threshold;     /* (B,H) or NULL */
+  float sm_scale;
+  float* delta;               /* (B,H,M) workspace, written */
+  float* dlog_lambda;         /* (B,H,N) workspace, written: gradient w.r.t. c */
+  float* dlog_fgate;          /* (B,H,N) written: gradient w.r.t. log_fgate */
+} fox_bwd_args;
+
+/*
+ * The four stages of the backward pass, in the order they must run on a stream:
+ *   fox_attn_bwd_delta : delta = rowsum(o * do)                     (_bwd_preprocess :902-943)
+ *   fox_attn_bwd_dkdv  : dk, dv, dlog_lambda[n] = -sum_i dS[i,n]   (_find_end_index_kernel :747-795 + _bwd_kv_kernel :956-1143)
+ *   fox_attn_bwd_dq    : dq, dlog_lambda[i+N-M] += sum_j dS[i,j]   (_find_start_index_kernel + _bwd_q_kernel :1156-1344)
+ *   fox_cumsum_bwd     : dlog_fgate from dlog_lambda                (:390-392)
+ * fox_attn_bwd runs all four (ForgettingAttention.backward :232-400).
+ */
+int fox_attn_bwd_delta(const fox_bwd_args* args, void* stream);
+int fox_attn_bwd_dkdv(const fox_bwd_args* args, void* stream);
+int fox_attn_bwd_dq(const fox_bwd_args* args, void* stream);
+int fox_attn_bwd(const fox_bwd_args* args, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FOX_ATTN_H */

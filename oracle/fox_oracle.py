@@ -1,0 +1,254 @@
+"""TEST INFRASTRUCTURE ONLY -- not part of the shipped operator.
+
+A plain-PyTorch restatement of the reference's materialised-mask Forgetting
+Attention, used as the checker for the HIP kernels.  Only tests, the smoke
+check and the CPU-baseline leg of the benchmark may import this module; the
+operator itself never does.
+
+Reference lines restated here (paths relative to the reference checkout):
+
+* ``src/forgetting_transformer/ops/forgetting_attention.py:1380-1404``
+  -- the pure-PyTorch Forgetting Attention inside ``test_op``: scores
+  ``q k^T * sm_scale`` plus the decay bias ``c[i + P_SEQ] - c[j]`` with
+  ``c = cumsum(log_fgate)``, a ``tril(diagonal=P_SEQ)`` causal mask, a
+  ``seq_start`` column mask, fp32 softmax, NaN -> 0 for rows with no valid
+  column, ``p @ v``, and gradients through ``torch.autograd``.
+* ``:111-127`` -- the operator's prologue: zero ``log_fgate`` left of
+  ``seq_start`` on a clone, then ``cumsum`` in fp32.
+* ``:91-102``  -- the ``"auto"`` pruning threshold.
+* ``:695-795`` -- the two block-boundary scans of Adaptive Computation Pruning
+  (restated in pure Python for small cases; the C restatement covers the
+  same scans for larger ones).
+* ``:902-943, 956-1143, 1156-1344, 390-392`` -- the manual backward
+  (``manual_backward`` below), written from the kernels' arithmetic.
+
+Pinned by (see tests/test_oracle_cpu.py): ``scaled_dot_product_attention`` with
+an additive mask, ``torch.logsumexp``, the ``g == 0`` and constant-``g``
+closed forms, ``torch.autograd.gradcheck`` in fp64, the identities
+``sum_n dc_n == 0`` and ``dg_l == sum_{i>=l} sum_{j<l} dS_ij``, brute force for
+the pruning boundaries, and the independent C restatement in ``fox_oracle.c``.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple, Union
+
+import torch
+
+__all__ = [
+    "cumulative_log_decay",
+    "auto_threshold",
+    "forgetting_attention_ref",
+    "forgetting_attention_ref_grads",
+    "manual_backward",
+    "find_start_index_ref",
+    "find_end_index_ref",
+]
+
+
+def cumulative_log_decay(log_fgate: torch.Tensor, seq_start: Optional[torch.Tensor],
+                         dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``c = cumsum(g)`` over the key axis with ``g[n < seq_start] = 0``.
+
+    ``log_fgate`` is head-first ``(B, H, N)``.  Follows
+    ``ops/forgetting_attention.py:117-127``.
+    """
+    g = log_fgate.to(dtype)
+    if seq_start is not None:
+        n = torch.arange(g.shape[-1], device=g.device)
+        g = torch.where(n[None, None, :] < seq_start[:, None, None], torch.zeros((), dtype=dtype, device=g.device), g)
+    return torch.cumsum(g, dim=-1)
+
+
+def auto_threshold(q: torch.Tensor, k: torch.Tensor, sm_scale: float) -> torch.Tensor:
+    """The ``"auto"`` threshold, ``(B, H)`` fp32, for head-first ``q``/``k``.
+
+    ``ops/forgetting_attention.py:95-102``: row L2 norms are taken in the
+    input dtype, the bound uses ``log(N)`` (keys, not queries) and a fixed
+    tolerance of ``-10``.
+    """
+    n_keys = k.shape[2]
+    max_q = torch.linalg.vector_norm(q, dim=-1).max(dim=-1).values
+    max_k = torch.linalg.vector_norm(k, dim=-1).max(dim=-1).values
+    ub = max_q * max_k * sm_scale
+    return (-(2 * ub + math.log(n_keys)) - 10).float()
+
+
+def _scores(q, k, c, seq_start, sm_scale):
+    """Masked scores ``(B, H, M, N)`` in the dtype of ``c``; -inf where invalid."""
+    M, N = q.shape[2], k.shape[2]
+    p_seq = N - M
+    s = torch.matmul(q, k.transpose(2, 3)) * sm_scale
+    s = s + (c[..., p_seq:, None] - c[..., None, :])
+    i = torch.arange(M, device=q.device)[:, None]
+    j = torch.arange(N, device=q.device)[None, :]
+    valid = (j <= i + p_seq)[None, None]
+    if seq_start is not None:
+        valid = valid & (j[None, None] >= seq_start[:, None, None, None])
+    return s.masked_fill(~valid, float("-inf")), valid
+
+
+def forgetting_attention_ref(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, log_fgate: torch.Tensor, *,
+    head_first: bool = False, seq_start: Optional[torch.Tensor] = None,
+    sm_scale: Optional[float] = None, compute_dtype: torch.dtype = torch.float32,
+    return_lse: bool = False, zero_gates_before_seq_start: bool = True,
+) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
+    """Materialised-mask Forgetting Attention (differentiable).
+
+    Mirrors ``ops/forgetting_attention.py:1380-1399`` with everything upcast
+    to ``compute_dtype`` (fp32 by default, fp64 for the tightest checks).
+    Rows with no valid column give ``out = 0`` and ``lse = -inf`` (``:1395-1397``
+    and the kernel's epilogue ``:679-685``).  The result is returned in
+    ``compute_dtype`` in the layout of the inputs.
+    """
+    if not head_first:
+        q, k, v = (x.transpose(1, 2) for x in (q, k, v))
+        log_fgate = log_fgate.transpose(1, 2)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    assert M <= N and log_fgate.shape == (B, H, N)
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    qf, kf, vf = (x.to(compute_dtype) for x in (q, k, v))
+    c = cumulative_log_decay(log_fgate, seq_start if zero_gates_before_seq_start else None, compute_dtype)
+    s, valid = _scores(qf, kf, c, seq_start, sm_scale)
+    any_valid = valid.any(dim=-1, keepdim=True)
+    # softmax with the NaN -> 0 convention for empty rows
+    s_safe = torch.where(any_valid, s, torch.zeros((), dtype=compute_dtype, device=s.device))
+    p = torch.softmax(s_safe, dim=-1)
+    p = torch.where(valid & any_valid, p, torch.zeros((), dtype=compute_dtype, device=s.device))
+    out = torch.matmul(p, vf)
+    if not head_first:
+        out = out.transpose(1, 2)
+    if return_lse:
+        lse = torch.logsumexp(s_safe, dim=-1)
+        lse = torch.where(any_valid[..., 0], lse, torch.full((), float("-inf"), dtype=compute_dtype, device=s.device))
+        return out, lse
+    return out
+
+
+def forgetting_attention_ref_grads(
+    q, k, v, log_fgate, dout, *, head_first=False, seq_start=None, sm_scale=None,
+    compute_dtype=torch.float32, bh_chunk: int = 0,
+):
+    """``(out, dq, dk, dv, dlog_fgate)`` through ``torch.autograd``
+    (``ops/forgetting_attention.py:1400-1404``), evaluated in chunks of
+    ``bh_chunk`` heads per batch element so long sequences fit in memory.
+    All results are in ``compute_dtype`` and in the layout of the inputs.
+    """
+    if not head_first:
+        q, k, v, dout = (x.transpose(1, 2) for x in (q, k, v, dout))
+        log_fgate = log_fgate.transpose(1, 2)
+    B, H = q.shape[:2]
+    step = bh_chunk if bh_chunk > 0 else H
+    outs, dqs, dks, dvs, dgs = [], [], [], [], []
+    for b in range(B):
+        ro, rq, rk, rv, rg = [], [], [], [], []
+        for h0 in range(0, H, step):
+            sl = slice(h0, min(H, h0 + step))
+            qq, kk, vv = (x[b:b + 1, sl].detach().to(compute_dtype).requires_grad_() for x in (q, k, v))
+            gg = log_fgate[b:b + 1, sl].detach().to(compute_dtype).requires_grad_()
+            ss = None if seq_start is None else seq_start[b:b + 1]
+            o = forgetting_attention_ref(qq, kk, vv, gg, head_first=True, seq_start=ss, sm_scale=sm_scale,
+                                         compute_dtype=compute_dtype)
+            o.backward(dout[b:b + 1, sl].to(compute_dtype))
+            ro.append(o.detach()); rq.append(qq.grad); rk.append(kk.grad); rv.append(vv.grad); rg.append(gg.grad)
+            del o, qq, kk, vv, gg
+        outs.append(torch.cat(ro, 1)); dqs.append(torch.cat(rq, 1)); dks.append(torch.cat(rk, 1))
+        dvs.append(torch.cat(rv, 1)); dgs.append(torch.cat(rg, 1))
+    out, dq, dk, dv, dg = (torch.cat(x, 0) for x in (outs, dqs, dks, dvs, dgs))
+    if not head_first:
+        out, dq, dk, dv = (x.transpose(1, 2) for x in (out, dq, dk, dv))
+        dg = dg.transpose(1, 2)
+    return out, dq, dk, dv, dg
+
+
+def manual_backward(q, k, v, log_fgate, dout, *, seq_start=None, sm_scale=None,
+                    compute_dtype=torch.float64, out_round_dtype: Optional[torch.dtype] = None):
+    """The kernels' hand-derived backward, head-first tensors only.
+
+    ``delta = rowsum(o * do)``            (``_bwd_preprocess`` ``:902-943``)
+    ``p = exp(s - lse)``; ``dp = do v^T``; ``ds = p (dp - delta)``
+    ``dv = p^T do``; ``dk = sm_scale ds^T q``   (``_bwd_kv_kernel`` ``:1073-1129``)
+    ``dq = sm_scale ds k``                       (``_bwd_q_kernel`` ``:1290-1333``)
+    ``dc[n] = -sum_i ds[i, n]`` (``:1122``) ``+ sum_j ds[n - P_SEQ, j]`` (``:1326, 1334-1344``)
+    ``dg = reverse inclusive cumsum(dc)``        (``:390-392``)
+
+    ``out_round_dtype`` optionally rounds ``o`` the way the operator stores it
+    before ``delta`` is formed.  Returns ``(out, lse, dq, dk, dv, dc, dg)``.
+    """
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    p_seq = N - M
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    qf, kf, vf, dof = (x.to(compute_dtype) for x in (q, k, v, dout))
+    c = cumulative_log_decay(log_fgate, seq_start, compute_dtype)
+    s, valid = _scores(qf, kf, c, seq_start, sm_scale)
+    any_valid = valid.any(dim=-1, keepdim=True)
+    zero = torch.zeros((), dtype=compute_dtype, device=s.device)
+    s_safe = torch.where(any_valid, s, zero)
+    lse = torch.logsumexp(s_safe, dim=-1, keepdim=True)
+    p = torch.where(valid & any_valid, torch.exp(s_safe - lse), zero)
+    out = p @ vf
+    o_used = out if out_round_dtype is None else out.to(out_round_dtype).to(compute_dtype)
+    delta = (o_used * dof).sum(-1, keepdim=True)
+    dp = dof @ vf.transpose(2, 3)
+    ds = p * (dp - delta)
+    dv = p.transpose(2, 3) @ dof
+    dk = sm_scale * (ds.transpose(2, 3) @ qf)
+    dq = sm_scale * (ds @ kf)
+    dc = -ds.sum(dim=2)
+    dc[..., p_seq:] += ds.sum(dim=3)
+    dg = torch.flip(torch.cumsum(torch.flip(dc, dims=[-1]), dim=-1), dims=[-1])
+    lse_out = torch.where(any_valid[..., 0], lse[..., 0], torch.full((), float("-inf"), dtype=compute_dtype, device=s.device))
+    return out, lse_out, dq, dk, dv, dc, dg
+
+
+def find_start_index_ref(c_row, threshold: float, M: int, N: int, block_m: int, block_n: int):
+    """Pure-Python restatement of ``_find_start_index_kernel`` (``:695-745``) for one
+    ``(b, h)`` row of ``c`` (a 1-D sequence of fp32 values): for each query block
+    the first key column (a multiple of ``block_n``) that may not be pruned.
+    """
+    p_seq = N - M
+    out = []
+    start = 0
+    c = [float(x) for x in c_row]
+    f32 = torch.float32
+    for m0 in range(0, M, block_m):
+        c_out = c[p_seq + m0]
+        while True:
+            col = min(N - 1, start + block_n - 1)
+            decay = float(torch.tensor(c_out, dtype=f32) - torch.tensor(c[col], dtype=f32))
+            if decay < threshold:
+                start += block_n
+            else:
+                break
+        out.append(start)
+    return out
+
+
+def find_end_index_ref(c_row, threshold: float, M: int, N: int, block_m: int, block_n: int, tight: bool = False):
+    """Pure-Python restatement of ``_find_end_index_kernel`` (``:747-795``): for each
+    key block the first query row (a multiple of ``block_m``, clamped to ``M``) from
+    which on the block may be pruned.  The reference reads ``c[row]`` without the
+    ``P_SEQ`` offset (``:783,789``); ``tight=True`` applies the offset, which prunes
+    more when ``M < N`` and is still safe.
+    """
+    p_seq = N - M if tight else 0
+    out = []
+    end = 0
+    c = [float(x) for x in c_row]
+    f32 = torch.float32
+    for n0 in range(0, N, block_n):
+        col = min(N - 1, n0 + block_n - 1)
+        while end < M:
+            row = min(end, M - 1) + p_seq
+            decay = float(torch.tensor(c[row], dtype=f32) - torch.tensor(c[col], dtype=f32))
+            if decay >= threshold:
+                end = min(end + block_m, M)
+            else:
+                break
+        out.append(end)
+    return out
