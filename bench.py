@@ -1,0 +1,322 @@
+#!/usr/bin/env python3
+"""Benchmark of the Forgetting Attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-extras] [--no-cpu-baseline]
+
+A step is one forward + backward pass of ``forgetting_attention`` over one batch
+of synthetic input already resident in HBM (forward only for c5).  The default
+workload is the long-context training-layer shape (B=4, T=16384, H=16, D=128,
+bf16, gate logits ~ N(3,1), head_first=False, no pruning); its FLOP count uses the
+reference's convention, fwd+bwd = 7*B*H*T^2*D.  One JSON line is printed.
+
+Besides the headline value the line carries
+  roofline     : the dominant kernel (dK/dV) timed alone with events on the launch
+                 stream, against the bf16 MFMA peak;
+  kernels      : the same for every stage of the path;
+  cpu_baseline : the PyTorch fp32 restatement of the reference's materialised-mask
+                 attention, forward only, on this host's cores, bounded to ~10 s;
+  acp          : pruned-tile fraction and speed-up of Adaptive Computation Pruning
+                 (thresholds "auto" and -10.0) on strongly decaying gates;
+  prefill      : chunked-prefill shape (M=128, N=32768, left padding), HBM GB/s.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT / "forgetting-transformer_amd"))
+sys.path.insert(0, str(ROOT))
+
+import torch  # noqa: E402
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: B, T(M), N, H, D, gate mean, gate std, head_first, fwd_only, seq_start
+    "c2": dict(B=4, M=512, N=512, H=12, D=64, mean=0.0, std=1.0, head_first=False, fwd_only=False, pad=False),
+    "c3": dict(B=4, M=16384, N=16384, H=16, D=128, mean=3.0, std=1.0, head_first=False, fwd_only=False, pad=False),
+    "c4": dict(B=4, M=16384, N=16384, H=16, D=128, mean=-1.0, std=2.0, head_first=False, fwd_only=False, pad=False),
+    "c5": dict(B=16, M=128, N=32768, H=16, D=128, mean=2.0, std=1.0, head_first=True, fwd_only=True, pad=True),
+}
+
+
+def synth(w, device, seed=0):
+    """Synthetic inputs of a workload, generated on the device from a fixed seed."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    B, M, N, H, D = w["B"], w["M"], w["N"], w["H"], w["D"]
+    shape_q = (B, H, M, D) if w["head_first"] else (B, M, H, D)
+    shape_k = (B, H, N, D) if w["head_first"] else (B, N, H, D)
+    shape_g = (B, H, N) if w["head_first"] else (B, N, H)
+    q = torch.randn(shape_q, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    k = torch.randn(shape_k, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    v = torch.randn(shape_k, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    logits = torch.randn(shape_g, generator=g, device=device, dtype=torch.float32) * w["std"] + w["mean"]
+    log_fgate = torch.nn.functional.logsigmoid(logits)
+    dout = torch.randn(shape_q, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    seq_start = None
+    if w["pad"]:
+        seq_start = torch.randint(0, 8192, (B,), generator=g, device=device, dtype=torch.long)
+    return q, k, v, log_fgate, dout, seq_start
+
+
+def flops_fwd(w):
+    # causal with offset: sum over rows of (row + P_SEQ + 1) columns, 4*D flops per (row, column)
+    M, N = w["M"], w["N"]
+    pairs = M * (N - M) + M * (M + 1) / 2
+    return 4.0 * w["B"] * w["H"] * pairs * w["D"]
+
+
+def time_steps(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def event_time(fn, iters, warmup=2):
+    """Average duration (s) of ``fn`` measured with events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) * 1e-3 / iters
+
+
+def stage_times(w, tensors, iters):
+    """Time every kernel of the path alone through the C ABI (launches go to torch's current stream)."""
+    from forgetting_transformer.ops import _lib
+    from forgetting_transformer.ops.forgetting_attention import _view
+
+    lib = _lib.load()
+    q, k, v, log_fgate, dout, seq_start = tensors
+    if not w["head_first"]:
+        q, k, v, dout = (x.transpose(1, 2) for x in (q, k, v, dout))
+        log_fgate = log_fgate.transpose(1, 2)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    dev = q.device
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    dims = _lib.Dims(B, H, M, N, D, _lib.DTYPE_BF16)
+    c = torch.empty((B, H, N), dtype=torch.float32, device=dev)
+    lse = torch.empty((B, H, M), dtype=torch.float32, device=dev)
+    o = torch.empty_like(q)
+    ss = None if seq_start is None else seq_start.data_ptr()
+    fwd = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), c.data_ptr(), lse.data_ptr(), ss, None,
+                       1.0 / math.sqrt(D), None)
+    out = {}
+
+    def scan():
+        _lib.check(lib.fox_cumsum_fwd(log_fgate.data_ptr(), *log_fgate.stride(), ss, c.data_ptr(), B, H, N, stream), "scan")
+
+    def f():
+        _lib.check(lib.fox_attn_fwd(C.byref(fwd), stream), "fwd")
+
+    scan()
+    out["cumsum_fwd"] = event_time(scan, iters)
+    out["fwd"] = event_time(f, iters)
+    if w["fwd_only"]:
+        return out
+    delta = torch.empty_like(lse)
+    dc = torch.empty_like(c)
+    dg = torch.empty_like(c)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    bwd = _lib.BwdArgs(dims, _view(q), _view(k), _view(v), _view(o), _view(dout), _view(dq), _view(dk), _view(dv),
+                       c.data_ptr(), lse.data_ptr(), ss, None, 1.0 / math.sqrt(D), delta.data_ptr(), dc.data_ptr(),
+                       dg.data_ptr())
+    for name, fn in (("bwd_delta", lib.fox_attn_bwd_delta), ("bwd_dkdv", lib.fox_attn_bwd_dkdv),
+                     ("bwd_dq", lib.fox_attn_bwd_dq)):
+        out[name] = event_time(lambda fn=fn, name=name: _lib.check(fn(C.byref(bwd), stream), name), iters)
+    out["cumsum_bwd"] = event_time(
+        lambda: _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg.data_ptr(), B, H, N, stream), "cumsum_bwd"), iters)
+    return out
+
+
+def cpu_baseline(budget_s=10.0):
+    """The reference's pure-PyTorch path (restated in oracle/), fp32 forward, B2 T256 H4 D64, on the host cores."""
+    from oracle.fox_oracle import forgetting_attention_ref
+
+    B, T, H, D = 2, 256, 4, 64
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn((B, T, H, D), generator=g) for _ in range(3))
+    log_fgate = torch.nn.functional.logsigmoid(torch.randn((B, T, H), generator=g))
+    cores = torch.get_num_threads()
+    fn = lambda: forgetting_attention_ref(q, k, v, log_fgate, sm_scale=1.0 / math.sqrt(D))
+    for _ in range(3):
+        fn()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while time.perf_counter() < t_end and len(times) < 2000:
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    flops = 4.0 * B * H * (T * (T + 1) / 2) * D
+    return {
+        "value": flops / med * 1e-12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"oracle/fox_oracle.py forward, fp32, B{B} T{T} H{H} D{D}, median of {len(times)} runs ({med * 1e3:.3f} ms), "
+                  "causal FLOPs 4*B*H*T(T+1)/2*D",
+    }
+
+
+def kept_fraction(start_index, M, N, block_m, block_n):
+    """Share of causal (query block, key block) tiles the forward visits, from the kernel's own bounds."""
+    p_seq = N - M
+    n_mt = start_index.shape[-1]
+    m0 = torch.arange(n_mt, device=start_index.device) * block_m
+    hi = torch.clamp(p_seq + m0 + block_m, max=N)
+    total = ((hi + block_n - 1) // block_n).sum().item() * start_index.shape[0] * start_index.shape[1]
+    kept = (((hi + block_n - 1) // block_n)[None, None, :] - start_index // block_n).sum().item()
+    return kept / total
+
+
+def acp_report(steps, warmup):
+    from forgetting_transformer import forgetting_attention
+    from forgetting_transformer.ops import _lib
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+
+    w = WORKLOADS["c4"]
+    q, k, v, log_fgate, dout, _ = synth(w, "cuda", seed=1)
+    q, k, v, log_fgate = (x.requires_grad_() for x in (q, k, v, log_fgate))
+    block_m, block_n, _, _ = _lib.tile_config(w["D"])
+    rep = {"workload": "B4 T16384 H16 D128 bf16 fwd+bwd, gate logits N(-1, 2)"}
+    base = None
+    ref_out = None
+    for name, thr in (("none", None), ("auto", "auto"), ("-10.0", -10.0)):
+        def step():
+            out = forgetting_attention(q, k, v, log_fgate, adaptive_threshold=thr)
+            out.backward(dout)
+            q.grad = k.grad = v.grad = log_fgate.grad = None
+        t = time_steps(step, steps, warmup)
+        with torch.no_grad():
+            out = forgetting_attention(q, k, v, log_fgate, adaptive_threshold=thr)
+        entry = {"ms_per_step": t * 1e3}
+        if thr is None:
+            base, ref_out = t, out
+        else:
+            with torch.no_grad():
+                _, _, si = ForgettingAttention.apply(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
+                                                     log_fgate.transpose(1, 2), None, True, None, thr, False, True)
+            kept = kept_fraction(si, w["M"], w["N"], block_m, block_n)
+            entry.update(pruned_tile_fraction=1.0 - kept, speedup_vs_none=base / t,
+                         max_abs_diff_vs_none=(out.float() - ref_out.float()).abs().max().item())
+        rep[name] = entry
+    return rep
+
+
+def prefill_report(steps, warmup):
+    from forgetting_transformer import forgetting_attention
+
+    w = WORKLOADS["c5"]
+    sets = [synth(w, "cuda", seed=10 + i) for i in range(3)]  # rotate so K/V do not sit in cache
+    idx = [0]
+
+    def step():
+        q, k, v, log_fgate, _, ss = sets[idx[0] % len(sets)]
+        idx[0] += 1
+        with torch.no_grad():
+            forgetting_attention(q, k, v, log_fgate, head_first=True, seq_start=ss)
+    t = time_steps(step, steps, warmup)
+    B, H, M, N, D = w["B"], w["H"], w["M"], w["N"], w["D"]
+    pad = torch.stack([s[5] for s in sets]).float().mean(0)  # mean left padding per batch row over the rotated sets
+    kv_bytes = (2.0 * H * (N - pad) * D * 2).sum().item()
+    other = 2 * B * H * M * D * 2 + B * H * N * 4 * 2
+    return {"workload": "B16 M128 N32768 H16 D128 bf16 forward, head_first, seq_start~U[0,8192)",
+            "ms_per_step": t * 1e3, "algorithmic_bytes": kv_bytes + other, "hbm_gbps": (kv_bytes + other) / t * 1e-9,
+            "frac_of_8TBps": (kv_bytes + other) / t * 1e-9 / PEAK_HBM_GBPS}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extras", action="store_true", help="skip the ACP and chunked-prefill reports")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ns = ap.parse_args()
+    if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py measures one GPU: Forgetting Attention never communicates (every (batch, head) pair is an "
+                 "independent problem), so a multi-GPU run would only replicate this measurement. Use --gpus 1.")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an AMD GPU (there is no CPU path for the operator)")
+
+    from forgetting_transformer import forgetting_attention
+
+    w = WORKLOADS[ns.workload]
+    tensors = synth(w, "cuda")
+    q, k, v, log_fgate, dout, seq_start = tensors
+    if not w["fwd_only"]:
+        q, k, v, log_fgate = (x.requires_grad_() for x in (q, k, v, log_fgate))
+
+    def step():
+        if w["fwd_only"]:
+            with torch.no_grad():
+                forgetting_attention(q, k, v, log_fgate, head_first=w["head_first"], seq_start=seq_start)
+        else:
+            out = forgetting_attention(q, k, v, log_fgate, head_first=w["head_first"], seq_start=seq_start)
+            out.backward(dout)
+            q.grad = k.grad = v.grad = log_fgate.grad = None
+
+    sec = time_steps(step, ns.steps, ns.warmup)
+    f_fwd = flops_fwd(w)
+    total = f_fwd if w["fwd_only"] else 3.5 * f_fwd  # bwd = 2.5 x fwd in the reference's convention
+    value = total / sec * 1e-12
+
+    stages = stage_times(w, tensors, max(3, ns.steps))
+    unit_flops = f_fwd / 2.0  # one causal matmul, B*H*T^2*D
+    kern_flops = {"fwd": 2 * unit_flops, "bwd_dkdv": 4 * unit_flops, "bwd_dq": 3 * unit_flops}
+    kernels = {}
+    for name, t in stages.items():
+        e = {"ms": t * 1e3}
+        if name in kern_flops:
+            e["tflops"] = kern_flops[name] / t * 1e-12
+            e["frac_of_peak"] = e["tflops"] / PEAK_BF16_TFLOPS
+        kernels[name] = e
+    dom = "fwd" if w["fwd_only"] else "bwd_dkdv"
+    roofline = {"kernel": dom, "bound": "mfma", "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": kernels[dom]["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
+                "avg_launch_ms": kernels[dom]["ms"]}
+
+    line = {
+        "metric": "fwd+bwd TFLOP/s & % bf16 MFMA peak, T=16k D=128; ACP speedup vs no-prune",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": ns.steps, "warmup": ns.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{ns.workload}: B{w['B']} M{w['M']} N{w['N']} H{w['H']} D{w['D']} bf16 "
+                               f"{'fwd' if w['fwd_only'] else 'fwd+bwd'}, gate logits N({w['mean']},{w['std']}), "
+                               f"head_first={w['head_first']}, no pruning",
+                   "flops_convention": "fwd 2*B*H*T^2*D, bwd 5*B*H*T^2*D (causal)"},
+        "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not ns.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+    if not ns.no_extras and ns.workload == "c3":
+        del q, k, v, log_fgate, dout, tensors
+        torch.cuda.empty_cache()
+        line["acp"] = acp_report(max(2, ns.steps // 2), 1)
+        torch.cuda.empty_cache()
+        line["prefill"] = prefill_report(max(5, ns.steps), 2)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -74,7 +74,7 @@ def auto_threshold(q: torch.Tensor, k: torch.Tensor, sm_scale: float) -> torch.T
     return (-(2 * ub + math.log(n_keys)) - 10).float()
 
 
-def _scores(q, k, c, seq_start, sm_scale):
+def _scores(q, k, c, seq_start, sm_scale, row_lo=None):
     """Masked scores ``(B, H, M, N)`` in the dtype of ``c``; -inf where invalid."""
     M, N = q.shape[2], k.shape[2]
     p_seq = N - M
@@ -85,6 +85,8 @@ def _scores(q, k, c, seq_start, sm_scale):
     valid = (j <= i + p_seq)[None, None]
     if seq_start is not None:
         valid = valid & (j[None, None] >= seq_start[:, None, None, None])
+    if row_lo is not None:
+        valid = valid & (j[None, None] >= row_lo[..., None])
     return s.masked_fill(~valid, float("-inf")), valid
 
 
@@ -92,14 +94,17 @@ def forgetting_attention_ref(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, log_fgate: torch.Tensor, *,
     head_first: bool = False, seq_start: Optional[torch.Tensor] = None,
     sm_scale: Optional[float] = None, compute_dtype: torch.dtype = torch.float32,
-    return_lse: bool = False, zero_gates_before_seq_start: bool = True,
+    return_lse: bool = False, zero_gates_before_seq_start: bool = True, row_lo: Optional[torch.Tensor] = None,
 ) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
     """Materialised-mask Forgetting Attention (differentiable).
 
     Mirrors ``ops/forgetting_attention.py:1380-1399`` with everything upcast
     to ``compute_dtype`` (fp32 by default, fp64 for the tightest checks).
     Rows with no valid column give ``out = 0`` and ``lse = -inf`` (``:1395-1397``
-    and the kernel's epilogue ``:679-685``).  The result is returned in
+    and the kernel's epilogue ``:679-685``).  ``row_lo`` ``(B, H, M)`` optionally
+    drops, per query row, every key column left of it: this is what Adaptive
+    Computation Pruning does when it starts a query block's key loop at
+    ``start_index`` (``:608-613``).  The result is returned in
     ``compute_dtype`` in the layout of the inputs.
     """
     if not head_first:
@@ -112,7 +117,7 @@ def forgetting_attention_ref(
         sm_scale = 1.0 / math.sqrt(D)
     qf, kf, vf = (x.to(compute_dtype) for x in (q, k, v))
     c = cumulative_log_decay(log_fgate, seq_start if zero_gates_before_seq_start else None, compute_dtype)
-    s, valid = _scores(qf, kf, c, seq_start, sm_scale)
+    s, valid = _scores(qf, kf, c, seq_start, sm_scale, row_lo)
     any_valid = valid.any(dim=-1, keepdim=True)
     # softmax with the NaN -> 0 convention for empty rows
     s_safe = torch.where(any_valid, s, torch.zeros((), dtype=compute_dtype, device=s.device))

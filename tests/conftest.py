@@ -39,6 +39,8 @@ def make_inputs(B, H, M, N, D, *, dtype=torch.bfloat16, device="cpu", seed=0, ga
     elif seq_start is not None:
         ss = torch.as_tensor(seq_start, dtype=torch.long)
     q, k, v, dout = (x.to(dtype) for x in (q, k, v, dout))
+    if dtype == torch.float64:
+        log_fgate = log_fgate.double()
     if not head_first:
         q, k, v, dout = (x.transpose(1, 2).contiguous() for x in (q, k, v, dout))
         log_fgate = log_fgate.transpose(1, 2).contiguous()

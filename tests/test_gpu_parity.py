@@ -1,0 +1,346 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI by the Python
+operator, against the oracle on the same seeded inputs.
+
+Tolerance (bf16): max |x - ref| <= 2e-2 * max(1, max|ref|) for out, dq, dk, dv,
+dlog_fgate, the bound BASELINE states ("max-abs error 2e-2 relative to output scale",
+with the scale floored at 1 so that a reference that is zero up to rounding -- a row with
+a single valid key has dS = 0 exactly -- does not turn rounding noise into a relative error).  The
+reference's own grid (fp16) uses its own bound, atol = 1e-2
+(ops/forgetting_attention.py:1416-1425).
+"""
+import ctypes as C
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from conftest import ROOT, make_inputs
+from oracle import fox_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def fa():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from forgetting_transformer import forgetting_attention
+    from forgetting_transformer.ops import _lib
+    _lib.load()  # fails loudly when the HIP library is missing
+    return forgetting_attention
+
+
+def rel_err(x, ref):
+    x, ref = x.float(), ref.float()
+    scale = max(1.0, ref.abs().max().item())    # "2e-2 * max(1, scale of x_ref)"
+    return (x - ref).abs().max().item() / scale
+
+
+def run_case(fa, B, H, M, N, D, *, dtype=torch.bfloat16, head_first=True, thr=None, sm_scale=None, tol=REL_TOL,
+             atol=None, **kw):
+    q, k, v, g, do, ss = make_inputs(B, H, M, N, D, dtype=dtype, device="cuda", head_first=head_first, **kw)
+    ref = O.forgetting_attention_ref_grads(q, k, v, g, do, head_first=head_first, seq_start=ss, sm_scale=sm_scale, bh_chunk=4)
+    q, k, v, g = (x.requires_grad_() for x in (q, k, v, g))
+    out = fa(q, k, v, g, head_first=head_first, seq_start=ss, sm_scale=sm_scale, adaptive_threshold=thr)
+    assert out.shape == q.shape and out.dtype == dtype
+    out.backward(do)
+    got = (out, q.grad, k.grad, v.grad, g.grad)
+    for name, x, r in zip(("out", "dq", "dk", "dv", "dlog_fgate"), got, ref):
+        assert torch.isfinite(x).all(), name
+        if atol is not None:
+            err = (x.float() - r.float()).abs().max().item()
+            assert err <= atol, f"{name}: abs err {err:.3e} > {atol}"
+        else:
+            e = rel_err(x, r)
+            assert e <= tol, f"{name}: rel err {e:.3e} > {tol}"
+    return got, ref, ss
+
+
+# --------------------------------------------------------------------------------------
+# committed golden vectors
+# --------------------------------------------------------------------------------------
+def test_golden_forward_backward(fa):
+    d = np.load(ROOT / "tests" / "golden" / "bwd_b2_h2_m72_n200_d32.npz")
+    t = lambda n, dt=torch.bfloat16: torch.from_numpy(d[n]).to("cuda").to(dt)
+    q, k, v, do = t("q"), t("k"), t("v"), t("dout")
+    g = t("log_fgate", torch.float32)
+    ss = torch.from_numpy(d["seq_start"]).cuda()
+    q, k, v, g = (x.requires_grad_() for x in (q, k, v, g))
+    out = fa(q, k, v, g, head_first=True, seq_start=ss, sm_scale=0.25)
+    out.backward(do)
+    for name, x in (("out", out), ("dq", q.grad), ("dk", k.grad), ("dv", v.grad), ("dlog_fgate", g.grad)):
+        assert rel_err(x, torch.from_numpy(d[name]).cuda()) <= REL_TOL, name
+    # batch row 1 starts at key 150 = query 22: queries 0..21 attend to nothing
+    assert (out[1, :, :22] == 0).all() and (q.grad[1, :, :22] == 0).all()
+    assert (k.grad[1, :, :150] == 0).all() and (v.grad[1, :, :150] == 0).all()
+    assert g.grad[1, :, :151].abs().max() <= 5e-3 * g.grad.abs().max()
+
+
+def test_golden_c1_shape(fa):
+    """BASELINE config 1 (B2 T256 H4 D64, sm_scale 1/8): same inputs rounded to bf16."""
+    d = np.load(ROOT / "tests" / "golden" / "c1_b2_t256_h4_d64.npz")
+    q, k, v = (torch.from_numpy(d[n]).cuda().bfloat16() for n in ("q", "k", "v"))
+    g = torch.from_numpy(d["log_fgate"]).cuda()
+    out = fa(q, k, v, g, sm_scale=1 / 8)
+    ref = O.forgetting_attention_ref(q, k, v, g, sm_scale=1 / 8)
+    assert rel_err(out, ref) <= REL_TOL
+    # and not far from the fp32-input golden output either (input rounding only)
+    assert rel_err(out, torch.from_numpy(d["out"]).cuda()) <= 5e-2
+
+
+# --------------------------------------------------------------------------------------
+# parity grid
+# --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("D", [16, 32, 64, 128])
+def test_config2_library_example(fa, D):
+    """BASELINE config 2: B4 T512 H12, bf16 fwd+bwd, (batch, time, head, dim) layout."""
+    run_case(fa, 4, 12, 512, 512, D, head_first=False, seed=D)
+
+
+@pytest.mark.parametrize("B,H,M,N,D", [(2, 2, 300, 300, 64), (1, 3, 129, 129, 128), (2, 2, 200, 457, 64), (1, 2, 64, 1000, 32),
+                                        (2, 1, 1, 777, 64), (1, 1, 1, 1, 16), (1, 2, 5, 5, 128), (1, 1, 127, 257, 16)])
+@pytest.mark.parametrize("seq", [None, "random"])
+def test_shapes_tails_and_offsets(fa, B, H, M, N, D, seq):
+    run_case(fa, B, H, M, N, D, seq_start=seq, seed=M + N)
+
+
+@pytest.mark.parametrize("seq", [[0, 0], [299, 5], [150, 299], [1, 128]])
+def test_seq_start_edges(fa, seq):
+    (out, dq, dk, dv, dg), _, ss = run_case(fa, 2, 2, 200, 300, 64, seq_start=seq, seed=5)
+    P = 100
+    for b, s in enumerate(seq):
+        empty = max(0, s - P)          # queries whose key position is left of seq_start
+        assert (out[b, :, :empty] == 0).all() and (dq[b, :, :empty] == 0).all()
+        assert (dk[b, :, :s] == 0).all() and (dv[b, :, :s] == 0).all()
+        assert dg[b, :, : s + 1].abs().max() <= 5e-3 * dg.abs().max()   # = sum of all dc, zero up to rounding
+
+
+@pytest.mark.parametrize("thr", [-10.0, "auto", "per_head", "per_bh", "zero_d"])
+@pytest.mark.parametrize("gates", [(0.0, 1.0), (-1.0, 2.0)])
+def test_adaptive_thresholds(fa, thr, gates):
+    """Thresholds low enough that the pruned attention mass is far below bf16 rounding:
+    results must match the unpruned oracle.  Covers the broadcast rules of :104-109."""
+    B, H = 2, 4
+    t = {"per_head": torch.tensor([-1000.0, -100.0, -40.0, -25.0]), "per_bh": torch.linspace(-60, -20, B * H).view(B, H),
+         "zero_d": torch.tensor(-30.0)}.get(thr, thr)
+    run_case(fa, B, H, 700, 1100, 64, thr=t, gate_mean=gates[0], gate_std=gates[1], qkv_std=0.5, seed=11)
+
+
+@pytest.mark.parametrize("thr", [-3.0, -0.5, 0.0])
+def test_aggressive_threshold_prunes_exactly_the_reported_tiles(fa, thr):
+    """A threshold that changes the result: the forward must equal the oracle with exactly the
+    key columns left of the kernel's reported start_index removed, and nothing else."""
+    from forgetting_transformer.ops import _lib
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    B, H, M, N, D = 2, 2, 600, 900, 64
+    bm, bn, _, _ = _lib.tile_config(D)
+    q, k, v, g, do, ss = make_inputs(B, H, M, N, D, device="cuda", seed=12, gate_mean=4.0, gate_std=1.0, seq_start=[0, 200])
+    q, k, v, g = (x.requires_grad_() for x in (q, k, v, g))
+    out, _, si = ForgettingAttention.apply(q, k, v, g, ss, True, None, thr, False, True)
+    assert (si % bn == 0).all() and (si > 0).any()
+    row_lo = si.repeat_interleave(bm, dim=-1)[..., :M]
+    ref = O.forgetting_attention_ref(q.detach(), k.detach(), v.detach(), g.detach(), head_first=True, seq_start=ss, row_lo=row_lo)
+    assert rel_err(out, ref) <= REL_TOL
+    full = O.forgetting_attention_ref(q.detach(), k.detach(), v.detach(), g.detach(), head_first=True, seq_start=ss)
+    assert rel_err(full, ref) > 1e-3          # the pruning really mattered at this threshold
+    out.backward(do)
+    for x in (q.grad, k.grad, v.grad, g.grad):
+        assert torch.isfinite(x).all()
+
+
+@pytest.mark.parametrize("sm_scale", [None, 0.5, 1.3])
+def test_sm_scale(fa, sm_scale):
+    run_case(fa, 1, 2, 260, 260, 64, sm_scale=sm_scale, qkv_std=0.5, seed=3)
+
+
+def test_fox_layer_views(fa):
+    """The FoX layer passes (B,H,T,D) views of (B,T,H*D) memory and a (B,H,T) view of
+    (B,T,H) gates with head_first=True (modeling_forgetting_transformer.py:318-346)."""
+    B, T, H, D = 2, 384, 4, 64
+    g = torch.Generator().manual_seed(0)
+    x = [torch.randn(B, T, H * D, generator=g).bfloat16().cuda() for _ in range(3)]
+    q, k, v = (t.view(B, T, H, D).transpose(1, 2).requires_grad_() for t in x)
+    gates = F.logsigmoid(torch.randn(B, T, H, generator=g).cuda()).transpose(1, 2).requires_grad_()
+    do = torch.randn(B, H, T, D, generator=g).bfloat16().cuda()
+    ss = torch.tensor([0, 100]).cuda()
+    out = fa(q, k, v, gates, head_first=True, seq_start=ss, sm_scale=1 / math.sqrt(D))
+    assert out.stride() == q.stride()                 # the un-permute on return stays free
+    out.backward(do)
+    ref = O.forgetting_attention_ref_grads(q.detach(), k.detach(), v.detach(), gates.detach(), do, head_first=True, seq_start=ss)
+    for x_, r in zip((out, q.grad, k.grad, v.grad, gates.grad), ref):
+        assert rel_err(x_, r) <= REL_TOL
+
+
+@pytest.mark.parametrize("Z,H,M,N,D", [(4, 2, 1020, 2098, 64), (4, 2, 1024, 2048, 128)])
+@pytest.mark.parametrize("gate_range", [(0, 5), (5, 10)])
+@pytest.mark.parametrize("has_seq_start", [True, False])
+@pytest.mark.parametrize("thr", [-10.0, None, "tensor"])
+def test_reference_grid(fa, Z, H, M, N, D, gate_range, has_seq_start, thr):
+    """The parameter grid, input distributions and tolerance of the reference's own test_op (:1360-1425)."""
+    t = torch.tensor([-1000.0, -100.0]) if thr == "tensor" else thr
+    run_case(fa, Z, H, M, N, D, dtype=torch.float16, qkv_std=0.5, gate_uniform=gate_range, sm_scale=0.5,
+             seq_start="random" if has_seq_start else None, thr=t, seed=24, atol=1e-2)
+
+
+# --------------------------------------------------------------------------------------
+# special cases and size-independent properties
+# --------------------------------------------------------------------------------------
+def test_zero_gates_are_plain_causal_attention(fa):
+    q, k, v, _, _, _ = make_inputs(2, 4, 512, 512, 64, device="cuda", seed=8)
+    g = torch.zeros(2, 4, 512, device="cuda")
+    out = fa(q, k, v, g, head_first=True)
+    ref = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True)
+    assert rel_err(out, ref) <= REL_TOL
+
+
+def test_log_normalizer_and_start_index_outputs(fa):
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    q, k, v, g, _, ss = make_inputs(2, 3, 300, 500, 64, device="cuda", seed=9, seq_start=[0, 350], gate_mean=-1, gate_std=2)
+    out, L, si = ForgettingAttention.apply(q, k, v, g, ss, True, 0.3, -6.0, True, True)
+    _, lse = O.forgetting_attention_ref(q, k, v, g, head_first=True, seq_start=ss, sm_scale=0.3, return_lse=True)
+    assert torch.equal(torch.isinf(L), torch.isinf(lse))
+    fin = ~torch.isinf(lse)
+    assert (L[fin] - lse[fin]).abs().max() < 2e-2
+    assert si.dtype == torch.long and si.shape == (2, 3, 3)
+
+
+def test_pruning_bounds_match_the_scan_bit_exactly(fa):
+    """first_block from the kernel's wave-parallel search == the reference's two-pointer scan
+    (restated in C) run on the kernel's own cumulative sums."""
+    import subprocess
+    from forgetting_transformer.ops import _lib
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    so = ROOT / "oracle" / "libfox_oracle.so"
+    if not so.exists():
+        subprocess.run(["make", "-C", str(ROOT / "oracle")], check=True, capture_output=True)
+    co = C.CDLL(str(so))
+    co.fox_oracle_find_start_index.argtypes = [C.c_void_p, C.c_float] + [C.c_int] * 4 + [C.c_void_p]
+    lib = _lib.load()
+    B, H, M, N, D = 2, 3, 1500, 4000, 64
+    bm, bn, _, _ = _lib.tile_config(D)
+    q, k, v, g, _, _ = make_inputs(B, H, M, N, D, device="cuda", seed=13, gate_mean=-1, gate_std=2)
+    thr = torch.tensor([[-5.0, -10.0, -40.0], [-1.0, -100.0, -20.0]])
+    _, _, si = ForgettingAttention.apply(q, k, v, g, None, True, None, thr, False, True)
+    c = torch.empty(B, H, N, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.fox_cumsum_fwd(g.data_ptr(), *g.stride(), None, c.data_ptr(), B, H, N, stream), "cumsum")
+    c = c.cpu().numpy()
+    for b in range(B):
+        for h in range(H):
+            row = np.ascontiguousarray(c[b, h])
+            exp = np.zeros((M + bm - 1) // bm, np.int64)
+            co.fox_oracle_find_start_index(row.ctypes.data_as(C.c_void_p), float(thr[b, h]), M, N, bm, bn,
+                                           exp.ctypes.data_as(C.c_void_p))
+            assert np.array_equal(si[b, h].cpu().numpy(), exp), (b, h)
+    assert (si > 0).any()
+
+
+def test_cumsum_kernels(fa):
+    from forgetting_transformer.ops import _lib
+    lib = _lib.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    B, H, N = 3, 5, 5000
+    g = F.logsigmoid(torch.randn(B, N, H, device="cuda") * 2 - 1).transpose(1, 2)   # strided (B,H,N) view
+    ss = torch.tensor([0, 1234, 4999], device="cuda")
+    c = torch.empty(B, H, N, device="cuda")
+    _lib.check(lib.fox_cumsum_fwd(g.data_ptr(), *g.stride(), ss.data_ptr(), c.data_ptr(), B, H, N, stream), "cumsum_fwd")
+    ref = O.cumulative_log_decay(g, ss, torch.float64)
+    assert (c.double() - ref).abs().max() <= 2e-7 * ref.abs().max()      # correctly rounded fp64 sums: half an ulp
+    assert (c[..., 1:] <= c[..., :-1]).all()                              # non-increasing, as the pruning bounds assume
+    assert (c[1, :, :1234] == 0).all()
+    dc = torch.randn(B, H, N, device="cuda")
+    dg = torch.empty_like(dc)
+    _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg.data_ptr(), B, H, N, stream), "cumsum_bwd")
+    ref = torch.flip(torch.cumsum(torch.flip(dc.double(), [-1]), -1), [-1])
+    assert (dg.double() - ref).abs().max() <= 1e-6 * ref.abs().max()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_auto_threshold_kernel(fa, dtype):
+    from forgetting_transformer.ops import _lib
+    from forgetting_transformer.ops.forgetting_attention import _view
+    lib = _lib.load()
+    B, H, M, N, D = 2, 3, 700, 1300, 64
+    q, k, _, _, _, _ = make_inputs(B, H, M, N, D, dtype=dtype, device="cuda", seed=17)
+    thr = torch.empty(B, H, device="cuda")
+    scratch = torch.empty(B, H, 2, dtype=torch.int32, device="cuda")
+    dims = _lib.Dims(B, H, M, N, D, 0 if dtype == torch.bfloat16 else 1)
+    qv, kv = _view(q), _view(k)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.fox_auto_threshold(C.byref(dims), C.byref(qv), C.byref(kv), 0.125, thr.data_ptr(), scratch.data_ptr(), stream), "auto")
+    ref = O.auto_threshold(q, k, 0.125)            # the reference's tensor arithmetic, same dtype roundings
+    ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10) * ref.abs().max().item()
+    assert (thr - ref).abs().max().item() <= 2 * ulp
+
+
+def test_bitwise_determinism(fa):
+    q, k, v, g, do, _ = make_inputs(2, 4, 1024, 1024, 128, device="cuda", seed=21, requires_grad=True)
+    res = []
+    for _ in range(2):
+        out = fa(q, k, v, g, head_first=True, adaptive_threshold="auto")
+        out.backward(do)
+        res.append([t.clone() for t in (out, q.grad, k.grad, v.grad, g.grad)])
+        q.grad = k.grad = v.grad = g.grad = None
+    for a, b in zip(*res):
+        assert torch.equal(a, b)          # no atomics anywhere on the path
+
+
+def test_linearity_in_values_and_upstream_gradient(fa):
+    q, k, v, g, do, _ = make_inputs(1, 2, 2048, 2048, 128, device="cuda", seed=22)
+    v2 = torch.randn_like(v)
+    f = lambda vv: fa(q, k, vv, g, head_first=True).float()
+    lhs = f((v.float() + v2.float()).bfloat16())
+    rhs = f(v) + f(v2)
+    assert rel_err(lhs, rhs) <= REL_TOL
+
+
+# --------------------------------------------------------------------------------------
+# BASELINE configs 3-5 at full size
+# --------------------------------------------------------------------------------------
+def _full_size_check(fa, B, H, T, D, mean, std, thr, pairs):
+    g_ = torch.Generator(device="cuda").manual_seed(3)
+    q, k, v = (torch.randn(B, T, H, D, generator=g_, device="cuda").bfloat16().requires_grad_() for _ in range(3))
+    gates = F.logsigmoid(torch.randn(B, T, H, generator=g_, device="cuda") * std + mean).requires_grad_()
+    do = torch.randn(B, T, H, D, generator=g_, device="cuda").bfloat16()
+    out = fa(q, k, v, gates, adaptive_threshold=thr)
+    out.backward(do)
+    got = (out, q.grad, k.grad, v.grad)
+    for x in got + (gates.grad,):
+        assert torch.isfinite(x).all()
+    # property: the gate gradient of position 0 is sum_n dc_n = 0
+    assert gates.grad[:, 0].abs().max() <= 1e-3 * max(1.0, gates.grad.abs().max().item())
+    for b, h in pairs:   # oracle on a few (batch, head) pairs: one pair needs a 1 GiB score matrix
+        sl = lambda x: x.detach()[b:b + 1, :, h:h + 1]
+        ref = O.forgetting_attention_ref_grads(sl(q), sl(k), sl(v), gates.detach()[b:b + 1, :, h:h + 1], sl(do))
+        for name, x, r in zip(("out", "dq", "dk", "dv"), got, ref):
+            assert rel_err(sl(x), r) <= REL_TOL, (name, b, h)
+        assert rel_err(gates.grad[b:b + 1, :, h:h + 1], ref[4]) <= REL_TOL, ("dlog_fgate", b, h)
+    return out.detach()
+
+
+def test_config3_long_context(fa):
+    _full_size_check(fa, 4, 16, 16384, 128, 3.0, 1.0, None, [(0, 0), (3, 15)])
+
+
+def test_config4_pruned(fa):
+    base = _full_size_check(fa, 4, 16, 16384, 128, -1.0, 2.0, None, [(1, 7)])
+    for thr in ("auto", -10.0):
+        out = _full_size_check(fa, 4, 16, 16384, 128, -1.0, 2.0, thr, [(1, 7)])
+        assert rel_err(out, base) <= 1e-3     # pruned mass <= e^-10: far below bf16 rounding
+
+
+def test_config5_chunked_prefill(fa):
+    B, H, M, N, D = 16, 16, 128, 32768, 128
+    g_ = torch.Generator(device="cuda").manual_seed(5)
+    q = torch.randn(B, H, M, D, generator=g_, device="cuda").bfloat16()
+    k = torch.randn(B, H, N, D, generator=g_, device="cuda").bfloat16()
+    v = torch.randn(B, H, N, D, generator=g_, device="cuda").bfloat16()
+    gates = F.logsigmoid(torch.randn(B, H, N, generator=g_, device="cuda") + 2.0)
+    ss = torch.randint(0, 8192, (B,), generator=g_, device="cuda")
+    out = fa(q, k, v, gates, head_first=True, seq_start=ss)
+    for b in range(B):
+        ref = O.forgetting_attention_ref(q[b:b + 1], k[b:b + 1], v[b:b + 1], gates[b:b + 1], head_first=True, seq_start=ss[b:b + 1])
+        assert rel_err(out[b:b + 1], ref) <= REL_TOL, b

@@ -1,0 +1,124 @@
+"""Host-side contract of the operator, checked without a GPU: the shared library
+loads and exports every symbol the public header declares, argument validation in
+the C ABI returns error codes before anything is launched, and the Python wrapper
+raises the reference's error types (ops/forgetting_attention.py:78-137, 447-448)."""
+import ctypes as C
+import re
+
+import pytest
+import torch
+
+from conftest import ROOT
+from forgetting_transformer import forgetting_attention
+from forgetting_transformer.ops import _lib
+from forgetting_transformer.ops.forgetting_attention import ForgettingAttention, maybe_contiguous
+
+
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "fox_attn.h").read_text()
+    declared = set(re.findall(r"^\s*(?:int|const char\*)\s+(fox_\w+)\s*\(", header, flags=re.M))
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.fox_version() >= 100
+
+
+def test_tile_config():
+    for d in (16, 32, 64, 128):
+        bm, bn, kbn, kbm = _lib.tile_config(d)
+        assert bm % 32 == 0 and bn % 32 == 0 and kbn % 32 == 0 and kbm % 32 == 0
+    with pytest.raises(RuntimeError, match="head dim"):
+        _lib.tile_config(48)
+
+
+def test_c_abi_rejects_bad_arguments_before_launching():
+    lib = _lib.load()
+    buf = (C.c_char * 4096)()
+    base = C.addressof(buf)
+    base += (-base) % 16
+    view = _lib.View(base, 64, 64, 64)
+
+    def fwd(dims, q=view, log_lambda=base):
+        a = _lib.FwdArgs(dims, q, view, view, view, log_lambda, base, None, None, 1.0, None)
+        return lib.fox_attn_fwd(C.byref(a), None)
+
+    assert fwd(_lib.Dims(1, 1, 8, 8, 48, 0)) == -1 and b"head dim" in lib.fox_last_error()
+    assert fwd(_lib.Dims(1, 1, 9, 8, 64, 0)) == -1 and b"M=9 > N=8" in lib.fox_last_error()
+    assert fwd(_lib.Dims(0, 1, 8, 8, 64, 0)) == -1
+    assert fwd(_lib.Dims(1, 1, 8, 8, 64, 7)) == -1 and b"dtype" in lib.fox_last_error()
+    assert fwd(_lib.Dims(1, 1, 8, 8, 64, 0), q=_lib.View(None, 64, 64, 64)) == -1 and b"q is NULL" in lib.fox_last_error()
+    assert fwd(_lib.Dims(1, 1, 8, 8, 64, 0), q=_lib.View(base + 2, 64, 64, 64)) == -2
+    assert fwd(_lib.Dims(1, 1, 8, 8, 64, 0), q=_lib.View(base, 64, 64, 12)) == -2 and b"strides" in lib.fox_last_error()
+    assert fwd(_lib.Dims(1, 1, 8, 8, 64, 0), log_lambda=None) == -1
+    assert lib.fox_attn_fwd(None, None) == -1
+    assert lib.fox_attn_bwd(None, None) == -1
+    assert lib.fox_cumsum_fwd(None, 1, 1, 1, None, base, 1, 1, 8, None) == -1
+    assert lib.fox_cumsum_bwd(base, base, 1, 1, 8, None) == -1 and b"alias" in lib.fox_last_error()
+    with pytest.raises(RuntimeError, match="code -1"):
+        _lib.check(-1, "x")
+
+
+def _cpu_inputs(B=2, T=8, H=2, D=64, dtype=torch.bfloat16):
+    q = torch.randn(B, T, H, D).to(dtype)
+    g = torch.nn.functional.logsigmoid(torch.randn(B, T, H))
+    return q, q.clone(), q.clone(), g
+
+
+def test_wrapper_error_contract():
+    q, k, v, g = _cpu_inputs()
+    with pytest.raises(AssertionError, match="Only torch.float16 or torch.bfloat16"):
+        forgetting_attention(q.float(), k, v, g)
+    with pytest.raises(AssertionError, match="head dims"):
+        forgetting_attention(q[..., :48], k[..., :48], v[..., :48], g)
+    with pytest.raises(AssertionError, match="float32"):
+        forgetting_attention(q, k, v, g.bfloat16())
+    with pytest.raises(AssertionError):
+        forgetting_attention(q, k, v, g[:, :-1])                       # wrong log_fgate shape
+    with pytest.raises(AssertionError, match="longer than the query"):
+        forgetting_attention(q, k[:, :4], v[:, :4], g[:, :4])          # M > N
+    with pytest.raises(AssertionError, match='"auto"'):
+        forgetting_attention(q, k, v, g, adaptive_threshold="automatic")
+    with pytest.raises(RuntimeError, match="broadcastable"):
+        forgetting_attention(q, k, v, g, adaptive_threshold=torch.zeros(3))
+    with pytest.raises(AssertionError):
+        forgetting_attention(q, k, v, g, seq_start=torch.zeros(5, dtype=torch.long))
+    with pytest.raises(AssertionError, match="feature size"):
+        forgetting_attention(q, k, v[..., :32], g)
+
+
+def test_no_cpu_fallback():
+    q, k, v, g = _cpu_inputs()
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        forgetting_attention(q, k, v, g)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        forgetting_attention(q, k, v, g, head_first=True, adaptive_threshold=-10.0, seq_start=torch.zeros(2, dtype=torch.long))
+
+
+def test_product_code_never_touches_the_oracle():
+    pkg = ROOT / "forgetting-transformer_amd"
+    for path in list(pkg.rglob("*.py")) + list(pkg.rglob("*.hip")) + list(pkg.rglob("*.hpp")):
+        text = path.read_text()
+        assert not re.search(r"\boracle\b", text), path
+        assert "_work/" not in text, path
+
+
+def test_maybe_contiguous_keeps_aligned_views():
+    x = torch.zeros(2, 16, 4 * 64, dtype=torch.bfloat16)
+    v = x.view(2, 16, 4, 64).transpose(1, 2)        # the (B,H,T,D) view the FoX layer passes (modeling_forgetting_transformer.py:318-320)
+    assert maybe_contiguous(v) is v
+    odd = torch.zeros(2, 2, 16, 65, dtype=torch.bfloat16)[..., :64]
+    assert maybe_contiguous(odd) is not odd and maybe_contiguous(odd).is_contiguous()
+    t = torch.zeros(2, 2, 64, 16, dtype=torch.bfloat16).transpose(2, 3)
+    assert maybe_contiguous(t).stride(-1) == 1
+
+
+def test_autograd_function_signature_matches_reference():
+    import inspect
+    params = list(inspect.signature(ForgettingAttention.forward).parameters)
+    assert params == ["ctx", "q", "k", "v", "log_fgate", "seq_start", "causal", "sm_scale", "adaptive_threshold",
+                      "return_log_normalizer", "return_start_index", "record_time_key", "record_attention_time",
+                      "record_find_index_time"]
+    sig = inspect.signature(forgetting_attention)
+    assert [p for p in sig.parameters] == ["q", "k", "v", "log_fgate", "head_first", "seq_start", "sm_scale", "adaptive_threshold"]
+    assert all(sig.parameters[p].kind is inspect.Parameter.KEYWORD_ONLY for p in ("head_first", "seq_start", "sm_scale", "adaptive_threshold"))

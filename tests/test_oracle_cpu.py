@@ -1,0 +1,327 @@
+"""Pins the oracle (oracle/fox_oracle.py and oracle/fox_oracle.c) on the CPU.
+
+The reference ships no golden vectors for this path, so every oracle function is
+pinned by something that does not share its code: a library routine it must
+reduce to, a closed form, an identity of the mathematics, brute force, or the
+other (independently written) restatement.
+"""
+import ctypes as C
+import math
+import subprocess
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from conftest import ROOT, make_inputs
+from oracle import fox_oracle as O
+
+torch.set_num_threads(4)
+
+
+# --------------------------------------------------------------------------------------
+# C restatement, loaded through ctypes
+# --------------------------------------------------------------------------------------
+@pytest.fixture(scope="session")
+def c_oracle():
+    so = ROOT / "oracle" / "libfox_oracle.so"
+    if not so.exists() or so.stat().st_mtime < (ROOT / "oracle" / "fox_oracle.c").stat().st_mtime:
+        subprocess.run(["make", "-C", str(ROOT / "oracle")], check=True, capture_output=True)
+    lib = C.CDLL(str(so))
+    return lib
+
+
+def _dptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def c_forward_backward(lib, q, k, v, g, do, seq_start, sm_scale):
+    """Run the C restatement on head-first tensors; returns numpy arrays."""
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    qd, kd, vd, dod = (np.ascontiguousarray(x.double().numpy()) for x in (q, k, v, do))
+    gf = np.ascontiguousarray(g.float().numpy())
+    ss = None if seq_start is None else np.ascontiguousarray(seq_start.numpy().astype(np.int64))
+    c = np.empty((B, H, N), np.float32)
+    lib.fox_oracle_cumsum(_dptr(gf), None if ss is None else _dptr(ss), _dptr(c), B, H, N)
+    out = np.empty((B, H, M, D)); lse = np.empty((B, H, M))
+    lib.fox_oracle_fwd.argtypes = [C.c_void_p] * 5 + [C.c_double] + [C.c_int] * 5 + [C.c_void_p] * 2
+    rc = lib.fox_oracle_fwd(_dptr(qd), _dptr(kd), _dptr(vd), _dptr(c), None if ss is None else _dptr(ss),
+                            sm_scale, B, H, M, N, D, _dptr(out), _dptr(lse))
+    assert rc == 0
+    dq = np.empty_like(qd); dk = np.empty_like(kd); dv = np.empty_like(vd)
+    dc = np.empty((B, H, N)); dg = np.empty((B, H, N))
+    lib.fox_oracle_bwd.argtypes = [C.c_void_p] * 5 + [C.c_double] + [C.c_int] * 5 + [C.c_void_p] * 8
+    rc = lib.fox_oracle_bwd(_dptr(qd), _dptr(kd), _dptr(vd), _dptr(c), None if ss is None else _dptr(ss), sm_scale,
+                            B, H, M, N, D, _dptr(out), _dptr(lse), _dptr(dod), _dptr(dq), _dptr(dk), _dptr(dv),
+                            _dptr(dc), _dptr(dg))
+    assert rc == 0
+    return dict(c=c, out=out, lse=lse, dq=dq, dk=dk, dv=dv, dc=dc, dg=dg)
+
+
+# --------------------------------------------------------------------------------------
+# forward: library pins
+# --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("B,H,M,N,D,ss", [(2, 4, 256, 256, 64, None), (2, 2, 37, 101, 16, None), (3, 2, 50, 80, 32, [0, 17, 60]),
+                                           (1, 1, 1, 33, 64, None)])
+def test_forward_matches_sdpa_with_additive_mask(B, H, M, N, D, ss):
+    q, k, v, g, _, seq = make_inputs(B, H, M, N, D, dtype=torch.float64, seed=1, seq_start=ss)
+    sm = 0.37
+    out, lse = O.forgetting_attention_ref(q, k, v, g, head_first=True, seq_start=seq, sm_scale=sm,
+                                          compute_dtype=torch.float64, return_lse=True)
+    # independent construction of the bias: explicit loops over the gate sums
+    c = torch.zeros(B, H, N, dtype=torch.float64)
+    for b in range(B):
+        s0 = 0 if seq is None else int(seq[b])
+        run = torch.zeros(H, dtype=torch.float64)
+        for n in range(N):
+            if n >= s0:
+                run = run + g[b, :, n]
+            c[b, :, n] = run
+    P = N - M
+    bias = torch.full((B, H, M, N), float("-inf"), dtype=torch.float64)
+    for i in range(M):
+        for b in range(B):
+            s0 = 0 if seq is None else int(seq[b])
+            lo, hi = s0, i + P
+            if lo <= hi:
+                bias[b, :, i, lo:hi + 1] = c[b, :, i + P, None] - c[b, :, lo:hi + 1]
+    empty = torch.isinf(bias).all(-1)
+    bias_safe = bias.clone()
+    bias_safe[empty] = 0.0
+    ref = F.scaled_dot_product_attention(q, k, v, attn_mask=bias_safe, scale=sm)
+    ref[empty] = 0.0
+    assert torch.allclose(out, ref, atol=1e-12, rtol=1e-10)
+    ref_lse = torch.logsumexp(q @ k.transpose(2, 3) * sm + bias, dim=-1)
+    assert torch.equal(torch.isinf(lse), empty)
+    assert torch.allclose(lse[~empty], ref_lse[~empty], atol=1e-12, rtol=1e-10)
+    assert (out[empty] == 0).all()
+
+
+def test_zero_gates_reduce_to_plain_causal_attention():
+    q, k, v, _, _, _ = make_inputs(2, 3, 64, 64, 32, dtype=torch.float64, seed=2)
+    g = torch.zeros(2, 3, 64, dtype=torch.float64)
+    out = O.forgetting_attention_ref(q, k, v, g, head_first=True, compute_dtype=torch.float64)
+    ref = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    assert torch.allclose(out, ref, atol=1e-12)
+
+
+def test_constant_gate_is_alibi():
+    B, H, M, N, D = 1, 2, 40, 72, 16
+    q, k, v, _, _, _ = make_inputs(B, H, M, N, D, dtype=torch.float64, seed=3)
+    slope = 0.3
+    g = torch.full((B, H, N), -slope, dtype=torch.float64)
+    out = O.forgetting_attention_ref(q, k, v, g, head_first=True, compute_dtype=torch.float64)
+    i = torch.arange(M)[:, None] + (N - M)
+    j = torch.arange(N)[None, :]
+    bias = torch.where(j <= i, -slope * (i - j).double(), torch.tensor(float("-inf"), dtype=torch.float64))
+    ref = F.scaled_dot_product_attention(q, k, v, attn_mask=bias)
+    assert torch.allclose(out, ref, atol=1e-12)
+
+
+def test_layouts_agree():
+    q, k, v, g, _, ss = make_inputs(2, 3, 20, 31, 16, dtype=torch.float64, seed=4, seq_start=[3, 0])
+    a = O.forgetting_attention_ref(q, k, v, g, head_first=True, seq_start=ss, compute_dtype=torch.float64)
+    b = O.forgetting_attention_ref(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), g.transpose(1, 2),
+                                   head_first=False, seq_start=ss, compute_dtype=torch.float64)
+    assert torch.equal(a, b.transpose(1, 2))
+
+
+def test_gates_left_of_seq_start_do_not_matter():
+    q, k, v, g, _, ss = make_inputs(2, 2, 24, 40, 16, dtype=torch.float64, seed=5, seq_start=[7, 19])
+    a = O.forgetting_attention_ref(q, k, v, g, head_first=True, seq_start=ss, compute_dtype=torch.float64)
+    b = O.forgetting_attention_ref(q, k, v, g, head_first=True, seq_start=ss, compute_dtype=torch.float64,
+                                   zero_gates_before_seq_start=False)  # the reference's test oracle does not zero them (:1386)
+    assert torch.allclose(a, b, atol=1e-12)
+
+
+# --------------------------------------------------------------------------------------
+# backward
+# --------------------------------------------------------------------------------------
+def test_gradcheck_fp64():
+    q, k, v, g, _, ss = make_inputs(1, 2, 5, 8, 16, dtype=torch.float64, seed=6, seq_start=[2], requires_grad=True)
+    fn = lambda q_, k_, v_, g_: O.forgetting_attention_ref(q_, k_, v_, g_, head_first=True, seq_start=ss, sm_scale=0.5,
+                                                           compute_dtype=torch.float64)
+    assert torch.autograd.gradcheck(fn, (q, k, v, g), eps=1e-6, atol=1e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("M,N,ss", [(48, 48, None), (30, 77, None), (30, 77, [0, 50, 76]), (1, 19, None)])
+def test_manual_backward_matches_autograd(M, N, ss):
+    B = 3 if ss else 2
+    q, k, v, g, do, seq = make_inputs(B, 2, M, N, 16, dtype=torch.float64, seed=7, seq_start=ss)
+    out, dq, dk, dv, dg = O.forgetting_attention_ref_grads(q, k, v, g, do, head_first=True, seq_start=seq, sm_scale=0.7,
+                                                           compute_dtype=torch.float64)
+    mo, ml, mdq, mdk, mdv, mdc, mdg = O.manual_backward(q, k, v, g, do, seq_start=seq, sm_scale=0.7)
+    for a, b in ((out, mo), (dq, mdq), (dk, mdk), (dv, mdv), (dg, mdg)):
+        assert torch.allclose(a, b, atol=1e-11, rtol=1e-9)
+    # identities of the mathematics
+    assert mdc.sum(-1).abs().max() < 1e-10          # sum_n dc_n = 0
+    if seq is not None:
+        for b in range(B):
+            assert mdg[b, :, : int(seq[b]) + 1].abs().max() < 1e-10   # dg_l = 0 for l <= seq_start
+    else:
+        assert mdg[..., 0].abs().max() < 1e-10
+
+
+def test_gate_gradient_closed_form():
+    """dg_l = sum over (rows at or after l) x (columns before l) of dS: only score
+    pairs that straddle position l contribute."""
+    B, H, M, N, D = 1, 2, 12, 20, 16
+    q, k, v, g, do, _ = make_inputs(B, H, M, N, D, dtype=torch.float64, seed=8)
+    P = N - M
+    _, _, _, _, _, _, mdg = O.manual_backward(q, k, v, g, do, sm_scale=0.4)
+    # dS by brute force
+    c = torch.cumsum(g, -1)
+    s = q @ k.transpose(2, 3) * 0.4 + (c[..., P:, None] - c[..., None, :])
+    i = torch.arange(M)[:, None] + P
+    j = torch.arange(N)[None, :]
+    s = s.masked_fill(j > i, float("-inf"))
+    p = torch.softmax(s, -1)
+    dp = do @ v.transpose(2, 3)
+    ds = p * (dp - (p * dp).sum(-1, keepdim=True))
+    for l in range(N):
+        rows = (torch.arange(M) + P) >= l
+        expect = ds[:, :, rows][..., :l].sum((-1, -2))
+        assert torch.allclose(mdg[..., l], expect, atol=1e-11)
+
+
+# --------------------------------------------------------------------------------------
+# the two restatements must agree
+# --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("B,H,M,N,D,ss", [(2, 4, 256, 256, 64, None), (2, 2, 61, 130, 32, [5, 100]), (1, 2, 1, 40, 16, None)])
+def test_c_restatement_matches_torch_restatement(c_oracle, B, H, M, N, D, ss):
+    q, k, v, g, do, seq = make_inputs(B, H, M, N, D, dtype=torch.float32, seed=9, seq_start=ss)
+    sm = 1.0 / math.sqrt(D)
+    r = c_forward_backward(c_oracle, q, k, v, g, do, seq, sm)
+    # cumsum: same fp32 running sum as torch on the CPU
+    c_t = O.cumulative_log_decay(g, seq, torch.float32)
+    assert np.allclose(r["c"], c_t.numpy(), atol=2e-5, rtol=1e-6)
+    g64 = torch.from_numpy(r["c"]).double()
+    g64 = torch.diff(g64, dim=-1, prepend=torch.zeros(B, H, 1, dtype=torch.float64))  # gates that reproduce the C cumsum exactly
+    out, lse = O.forgetting_attention_ref(q, k, v, g64, head_first=True, seq_start=None if seq is None else seq,
+                                          sm_scale=sm, compute_dtype=torch.float64, return_lse=True,
+                                          zero_gates_before_seq_start=False)
+    assert np.allclose(r["out"], out.numpy(), atol=1e-9)
+    fin = ~torch.isinf(lse)
+    assert np.array_equal(np.isinf(r["lse"]), ~fin.numpy())
+    assert np.allclose(r["lse"][fin.numpy()], lse[fin].numpy(), atol=1e-9)
+    _, dq, dk, dv, dg = O.forgetting_attention_ref_grads(q, k, v, g64, do, head_first=True, seq_start=seq, sm_scale=sm,
+                                                         compute_dtype=torch.float64)
+    for name, t in (("dq", dq), ("dk", dk), ("dv", dv)):
+        assert np.allclose(r[name], t.numpy(), atol=1e-9), name
+    # gate gradient: compare where gates matter (right of seq_start); left of it both are 0
+    assert np.allclose(r["dg"], dg.numpy(), atol=1e-8)
+    assert abs(r["dc"].sum(-1)).max() < 1e-9
+
+
+# --------------------------------------------------------------------------------------
+# Adaptive Computation Pruning bounds
+# --------------------------------------------------------------------------------------
+def _brute_start(c, thr, M, N, bm, bn):
+    """First key block of each query block that holds an entry with decay >= thr (causal part only)."""
+    P = N - M
+    out = []
+    for m0 in range(0, M, bm):
+        rows = range(m0, min(M, m0 + bm))
+        first = None
+        for t in range(0, (P + m0) // bn + 1):
+            cols = range(t * bn, min(N, t * bn + bn))
+            if any(np.float32(c[P + i]) - np.float32(c[j]) >= np.float32(thr) for i in rows for j in cols):
+                first = t
+                break
+        out.append((first if first is not None else (P + m0) // bn) * bn)
+    return out
+
+
+@pytest.mark.parametrize("M,N,bm,bn,thr", [(64, 64, 16, 8, -3.0), (50, 120, 16, 16, -6.0), (128, 128, 128, 64, -10.0),
+                                            (33, 97, 8, 32, -1.0), (40, 40, 8, 8, 0.0)])
+def test_start_index_scan_is_exact(c_oracle, M, N, bm, bn, thr):
+    g = torch.Generator().manual_seed(M * 1000 + N)
+    c = torch.cumsum(F.logsigmoid(torch.randn(N, generator=g) * 2 - 1), 0).float()
+    py = O.find_start_index_ref(c, thr, M, N, bm, bn)
+    out = np.zeros(len(py), np.int64)
+    cn = np.ascontiguousarray(c.numpy())
+    c_oracle.fox_oracle_find_start_index.argtypes = [C.c_void_p, C.c_float] + [C.c_int] * 4 + [C.c_void_p]
+    c_oracle.fox_oracle_find_start_index(_dptr(cn), thr, M, N, bm, bn, _dptr(out))
+    assert list(out) == py
+    # because c is non-increasing the scan equals brute force over every entry of every rectangle
+    assert py == _brute_start(cn, thr, M, N, bm, bn)
+    # safety: everything left of the bound is below the threshold
+    P = N - M
+    for blk, start in enumerate(py):
+        for i in range(blk * bm, min(M, blk * bm + bm)):
+            for j in range(0, min(start, P + i + 1)):
+                assert cn[P + i] - cn[j] < thr
+
+
+@pytest.mark.parametrize("M,N,bm,bn,thr", [(64, 64, 16, 8, -3.0), (50, 120, 16, 16, -6.0), (128, 128, 32, 128, -10.0)])
+def test_end_index_scan_is_safe(c_oracle, M, N, bm, bn, thr):
+    g = torch.Generator().manual_seed(M * 77 + N)
+    c = torch.cumsum(F.logsigmoid(torch.randn(N, generator=g) * 2 - 1), 0).float()
+    cn = np.ascontiguousarray(c.numpy())
+    P = N - M
+    c_oracle.fox_oracle_find_end_index.argtypes = [C.c_void_p, C.c_float] + [C.c_int] * 5 + [C.c_void_p]
+    for tight in (0, 1):
+        py = O.find_end_index_ref(c, thr, M, N, bm, bn, tight=bool(tight))
+        out = np.zeros(len(py), np.int64)
+        c_oracle.fox_oracle_find_end_index(_dptr(cn), thr, M, N, bm, bn, tight, _dptr(out))
+        assert list(out) == py
+        for blk, end in enumerate(py):
+            for j in range(blk * bn, min(N, blk * bn + bn)):
+                for i in range(end, M):
+                    if j <= P + i:
+                        assert cn[P + i] - cn[j] < thr
+    loose = O.find_end_index_ref(c, thr, M, N, bm, bn, tight=False)
+    tight_ = O.find_end_index_ref(c, thr, M, N, bm, bn, tight=True)
+    assert all(t <= l for t, l in zip(tight_, loose))   # the reference's bound only ever prunes less
+
+
+def test_pruned_mass_is_bounded_by_the_auto_threshold():
+    """With thr = -(2 ub + log N) - 10 the attention mass of pruned entries is <= e^-10 per row."""
+    B, H, T, D = 1, 2, 96, 16
+    q, k, v, g, _, _ = make_inputs(B, H, T, T, D, dtype=torch.float64, seed=11, gate_mean=-1.0, gate_std=2.0)
+    sm = 1 / math.sqrt(D)
+    thr = O.auto_threshold(q, k, sm).double()
+    c = torch.cumsum(g, -1)
+    decay = c[..., :, None] - c[..., None, :]
+    s = q @ k.transpose(2, 3) * sm + decay
+    mask = torch.tril(torch.ones(T, T, dtype=torch.bool))
+    s = s.masked_fill(~mask, float("-inf"))
+    p = torch.softmax(s, -1)
+    pruned = (decay < thr[..., None, None]) & mask
+    assert pruned.any()
+    assert (p * pruned).sum(-1).max() <= math.exp(-10)
+    out_full = p @ v
+    out_pruned = (p * ~pruned) @ v
+    assert (out_full - out_pruned).abs().max() <= 2 * math.exp(-10) * v.abs().max()
+
+
+def test_auto_threshold_closed_form():
+    """README.md:196-209 of the reference states the same recipe with explicit norms."""
+    q, k, _, _, _, _ = make_inputs(2, 3, 17, 29, 32, dtype=torch.float32, seed=12)
+    sm = 1 / math.sqrt(32)
+    thr = O.auto_threshold(q, k, sm)
+    qn = q.double().pow(2).sum(-1).sqrt().amax(-1)
+    kn = k.double().pow(2).sum(-1).sqrt().amax(-1)
+    expect = -(2 * qn * kn / math.sqrt(32) + math.log(29)) - 10
+    assert torch.allclose(thr.double(), expect, atol=1e-4)
+
+
+# --------------------------------------------------------------------------------------
+# committed golden vectors
+# --------------------------------------------------------------------------------------
+def test_golden_fixture_is_reproduced():
+    data = np.load(ROOT / "tests" / "golden" / "c1_b2_t256_h4_d64.npz")
+    q, k, v, g = (torch.from_numpy(data[n]) for n in ("q", "k", "v", "log_fgate"))
+    out, lse = O.forgetting_attention_ref(q, k, v, g, sm_scale=1 / 8, return_lse=True)
+    assert np.allclose(out.numpy(), data["out"], atol=1e-6)
+    assert np.allclose(lse.numpy(), data["lse"], atol=1e-5)
+    # and against the other restatement, which shares no code with the one that wrote the file
+    ref = F.scaled_dot_product_attention
+    c = torch.cumsum(g.transpose(1, 2).double(), -1)
+    T = q.shape[1]
+    bias = (c[..., :, None] - c[..., None, :]).masked_fill(~torch.tril(torch.ones(T, T, dtype=torch.bool)), float("-inf"))
+    o2 = ref(q.transpose(1, 2).double(), k.transpose(1, 2).double(), v.transpose(1, 2).double(), attn_mask=bias, scale=1 / 8)
+    assert np.allclose(o2.transpose(1, 2).numpy(), data["out"], atol=1e-5)
