@@ -52,10 +52,12 @@ def build(jobs: int = 4, force: bool = True) -> Path:
             return LIB_PATH
     with concurrent.futures.ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
         objs = list(ex.map(_compile, SOURCES))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB_PATH)]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--no-undefined", *map(str, objs), "-o", str(LIB_PATH)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stderr}")
+    import ctypes
+    ctypes.CDLL(str(LIB_PATH), mode=ctypes.RTLD_GLOBAL | getattr(os, "RTLD_NOW", 2))  # every symbol must resolve
     return LIB_PATH
 
 

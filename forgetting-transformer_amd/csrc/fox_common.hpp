@@ -152,6 +152,49 @@ struct TileLoader {
   }
 };
 
+// ---------------------------------------------------------------------------
+// HBM -> LDS tile loader without registers: buffer loads with the LDS bit.  Each
+// wave instruction moves 64 x 16 bytes into a contiguous 1 KiB block of LDS (slot
+// of lane l = block base + 16*l, whatever address the lane reads from), so the
+// swizzle is applied on the global side: the lane that owns LDS slot (row, c')
+// fetches chunk c' ^ swz(row) of that row.  Rows at or beyond row_limit lie
+// outside the buffer resource and read as zero.  The caller waits for vmcnt(0) and
+// a barrier before the tile is read.
+// ---------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+__device__ inline void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), other counters untouched
+
+template <int D, int ROWS>
+struct DirectTileLoader {
+  static constexpr int CH = D / 8;
+  static constexpr int NBLK = ROWS * CH / 64;  // 1 KiB blocks per tile
+  static constexpr int PER = (NBLK + 3) / 4;   // blocks per wave (4 waves)
+  static_assert(ROWS * CH % 64 == 0, "tile must be a whole number of 1 KiB blocks");
+  int voff[PER];
+  int wave;
+
+  __device__ inline DirectTileLoader(int64_t row_stride, int wave_, int lane) : wave(wave_) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int pos = (wave + 4 * j) * 64 + lane;
+      const int row = pos / CH, cp = pos % CH;
+      voff[j] = (int)(row * row_stride * 2) + ((cp ^ Tile<D>::swz(row)) << 4);
+    }
+  }
+  __device__ inline void issue(const uint16_t* base, int64_t row_stride, int row0, int row_limit, char* tile) const {
+    const uint16_t* p = base + (int64_t)row0 * row_stride;
+    const int64_t bytes = row_limit > row0 ? ((int64_t)(row_limit - 1 - row0) * row_stride + D) * 2 : 0;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, (int)bytes, 0x00020000);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int blk = wave + 4 * j;
+      if (NBLK % 4 == 0 || blk < NBLK)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(tile + blk * 1024), 16, voff[j], 0, 0, 0);
+    }
+  }
+};
+
 // Operand held in registers for a whole kernel: lane (g, i) keeps row (row0 + i),
 // elements 16*kk + 8*g .. +7 for every k-step kk.  Rows >= row_limit are zero.
 template <int D>

@@ -5,30 +5,128 @@
 // S^T = K Q^T (32x32x16 MFMA).  With the scores transposed, lane (g, i) holds one
 // query row i and 16 key columns per 32-column block, so the online-softmax row
 // statistics are lane-local plus one exchange between the two 32-lane halves, and
-// the probabilities are already laid out as the B operand of O^T = V^T P^T.  K and
-// V tiles are staged through LDS; V^T is read with the transposing LDS load.
+// the probabilities are already laid out as the B operand of O^T = V^T P^T.
+//
+// K and V tiles of 64 keys go from HBM straight into LDS (buffer loads with the
+// LDS bit: no registers, no ds_write; out-of-range rows read as zero), into two
+// alternating buffers, so the loads of the next tile fly while the current one is
+// consumed and there is one barrier per tile.  V^T is read with the transposing
+// LDS load.
+//
+// Key tiles are walked from the diagonal backwards.  Under a forget gate the
+// scores shrink with distance, so the running row maximum is set by the first
+// tiles; it is only raised when a tile exceeds it by more than 2^8, which keeps
+// every exponent <= 8 (exact in fp32/bf16 terms, the factor cancels in o = acc/l)
+// and makes the rescale of the accumulator a rare, wave-uniform branch.
 //
 // The decay bias enters relative to c_ref = c[first query row of the tile]:
 //   x = (q.k) * sm_scale*log2e - (c_n - c_ref)*log2e          (per score)
 // and the row term (c_m - c_ref)*log2e, constant along a row, is only added to the
 // stored log-normaliser.  Columns left of seq_start (and beyond N) get
 // (c_n - c_ref) = +inf, which makes x = -inf without a compare in the loop; only
-// tiles crossing the diagonal run the causal compare.
+// tiles crossing the diagonal run the causal compare (separate code path).
 #include "fox_common.hpp"
 #include "fox_kernels.hpp"
 
 namespace fox {
 
+constexpr float kLazyMaxLog2 = 8.0f;
+
+template <typename Tr, int D>
+__device__ inline void fwd_tile(const char* k_tile, const char* v_tile, const float* cn_s, const u32x4 (&qreg)[D / 16],
+                                f32x16 (&oacc)[(D + 31) / 32], float& m_i, float& l_i, int n0, int a_m, float qk_scale,
+                                int lane, bool diag) {
+  constexpr int BN = kFwdBN, KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
+  const int g = lane >> 5, i = lane & 31;
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  // S^T = K Q^T
+  f32x16 s[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    u32x4 ka[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) ka[kk] = lds_row_operand<D>(k_tile, 32 * nb + i, 2 * kk + g);
+    s[nb] = Tr::mfma32(ka[0], qreg[0], zero);
+#pragma unroll
+    for (int kk = 1; kk < KK; ++kk) s[nb] = Tr::mfma32(ka[kk], qreg[kk], s[nb]);
+  }
+
+  // scores in the log2 domain and their maximum
+  float mloc = -INFINITY;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const f32x4 cn = *reinterpret_cast<const f32x4*>(&cn_s[32 * nb + 8 * q4 + 4 * g]);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int r = 4 * q4 + t;
+        s[nb][r] = fmaf(s[nb][r], qk_scale, -cn[t]);
+      }
+    }
+  }
+  if (diag) {  // causal compare, only on tiles that cross the diagonal
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int n = n0 + 32 * nb + c_row(r, g);
+        s[nb][r] = (n > a_m) ? -INFINITY : s[nb][r];
+      }
+  }
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, s[nb][r]);
+  mloc = half_max(mloc);
+  const bool raise = mloc > m_i + kLazyMaxLog2;
+  if (__any(raise)) {  // rare: rescale what has been accumulated so far
+    const float m_new = raise ? mloc : m_i;
+    const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+    m_i = m_new;
+    l_i *= alpha;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+  }
+  float rsum = 0.f;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float p = __builtin_amdgcn_exp2f(s[nb][r] - m_i);
+      s[nb][r] = p;
+      rsum += p;
+    }
+  l_i += rsum;  // per-lane partial sum; the two halves are added in the epilogue
+
+  // O^T += V^T P^T
+#pragma unroll
+  for (int sl = 0; sl < BN / 16; ++sl) {
+    const u32x4 pb = pack8<Tr>(s[sl >> 1], 8 * (sl & 1));
+    u32x4 va[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) va[db] = lds_col_operand<D>(v_tile, 16 * sl, db, lane);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) oacc[db] = Tr::mfma32(va[db], pb, oacc[db]);
+  }
+}
+
 template <typename Tr, int D>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
-  constexpr int BM = kFwdBM, BN = kFwdBN, NT = 256;
-  constexpr int KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
+  constexpr int BM = kFwdBM, BN = kFwdBN;
+  constexpr int KK = D / 16, DB = (D + 31) / 32;
   static_assert(BM == 128, "four waves of 32 rows");
-  __shared__ __align__(16) char k_tile[BN * D * 2];
-  __shared__ __align__(16) char v_tile[BN * D * 2];
-  __shared__ __align__(16) float cn_s[BN];
+  __shared__ __align__(16) char k_tile0[BN * D * 2];
+  __shared__ __align__(16) char k_tile1[BN * D * 2];
+  __shared__ __align__(16) char v_tile0[BN * D * 2];
+  __shared__ __align__(16) char v_tile1[BN * D * 2];
+  __shared__ __align__(16) float cn_s0[BN];
+  __shared__ __align__(16) float cn_s1[BN];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, i = lane & 31;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), g = lane >> 5, i = lane & 31;
   int bh, mt;
   decode_block(blockIdx.x, a.n_mtiles, a.B * a.H, bh, mt);
   const int b = bh / a.H, h = bh % a.H;
@@ -54,6 +152,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   }
   lo = (lo / BN) * BN;
   if (a.first_block && tid == 0) a.first_block[(int64_t)bh * a.n_mtiles + mt] = lo / BN;
+  const int n_tiles = (hi - lo + BN - 1) / BN;  // walked from the last (diagonal) tile down to lo
 
   const int m = m0 + 32 * wave + i;  // this lane's query row
   const int a_m = p_seq + m;
@@ -69,87 +168,41 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
-  float m_i = -INFINITY, l_i = 0.f;
+  float m_i = -3.0e38f, l_i = 0.f;  // finite floor: a row that has seen no valid key yet yields exp2(-inf) = 0
 
-  TileLoader<D, BN, NT> kl, vl;
+  const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
   float cn_pref = 0.f;
-  auto prefetch = [&](int n0) {
-    kl.load(kp, a.k.st, n0, N, tid);
-    vl.load(vp, a.v.st, n0, N, tid);
+  auto issue = [&](int n0, char* kt, char* vt) {
+    kld.issue(kp, a.k.st, n0, N, kt);
+    vld.issue(vp, a.v.st, n0, N, vt);
     if (tid < BN) {
       const int n = n0 + tid;
       cn_pref = (n < N && n >= seq) ? (c_row[n] - c_ref) * kLog2e : INFINITY;
     }
   };
-  if (lo < hi) prefetch(lo);
+  auto compute = [&](int n0, const char* kt, const char* vt, const float* cn) {
+    if (n0 > a_w0 + 31) return;  // tile entirely above this wave's rows
+    fwd_tile<Tr, D>(kt, vt, cn, qreg, oacc, m_i, l_i, n0, a_m, qk_scale, lane, n0 + BN - 1 > a_w0);
+  };
 
-  for (int n0 = lo; n0 < hi; n0 += BN) {
-    __syncthreads();  // every wave is done with the previous tile
-    kl.store(k_tile, tid);
-    vl.store(v_tile, tid);
-    if (tid < BN) cn_s[tid] = cn_pref;
+  if (n_tiles > 0) {
+    issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
+    if (tid < BN) cn_s0[tid] = cn_pref;
+  }
+  for (int t = n_tiles - 1; t >= 0; t -= 2) {
+    // even step: consume buffers 0, fill buffers 1
+    wait_vmem_all();
     __syncthreads();
-    if (n0 + BN < hi) prefetch(n0 + BN);
-    if (n0 > a_w0 + 31) continue;  // tile entirely above this wave's rows
-    const bool diag = n0 + BN - 1 > a_w0;
-
-    // S^T = K Q^T
-    f32x16 s[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[nb][r] = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk)
-        s[nb] = Tr::mfma32(lds_row_operand<D>(k_tile, 32 * nb + i, 2 * kk + g), qreg[kk], s[nb]);
-    }
-
-    // scores in the log2 domain, running max
-    float mloc = -INFINITY;
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const f32x4 cn = *reinterpret_cast<const f32x4*>(&cn_s[32 * nb + 8 * q4 + 4 * g]);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int r = 4 * q4 + t;
-          float x = fmaf(s[nb][r], qk_scale, -cn[t]);
-          if (diag) {
-            const int n = n0 + 32 * nb + 8 * q4 + 4 * g + t;
-            x = (n > a_m) ? -INFINITY : x;
-          }
-          s[nb][r] = x;
-          mloc = fmaxf(mloc, x);
-        }
-      }
-    }
-    mloc = half_max(mloc);
-    const float m_use = fmaxf(fmaxf(m_i, mloc), -3.0e38f);  // finite even when the row is still empty
-    const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
-    float rsum = 0.f;
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = __builtin_amdgcn_exp2f(s[nb][r] - m_use);
-        s[nb][r] = p;
-        rsum += p;
-      }
-    l_i = l_i * alpha + rsum;  // per-lane partial sum; the two halves are added in the epilogue
-    m_i = m_use;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-
-    // O^T += V^T P^T
-#pragma unroll
-    for (int sl = 0; sl < BN / 16; ++sl) {
-      const u32x4 pb = pack8<Tr>(s[sl >> 1], 8 * (sl & 1));
-#pragma unroll
-      for (int db = 0; db < DB; ++db) oacc[db] = Tr::mfma32(lds_col_operand<D>(v_tile, 16 * sl, db, lane), pb, oacc[db]);
-    }
+    if (t >= 1) issue(lo + (t - 1) * BN, k_tile1, v_tile1);
+    compute(lo + t * BN, k_tile0, v_tile0, cn_s0);
+    if (t < 1) break;
+    if (tid < BN) cn_s1[tid] = cn_pref;
+    // odd step: consume buffers 1, fill buffers 0
+    wait_vmem_all();
+    __syncthreads();
+    if (t >= 2) issue(lo + (t - 2) * BN, k_tile0, v_tile0);
+    compute(lo + (t - 1) * BN, k_tile1, v_tile1, cn_s1);
+    if (t >= 2 && tid < BN) cn_s0[tid] = cn_pref;
   }
 
   // epilogue
@@ -172,6 +225,15 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     if (g == 0) a.lse[(int64_t)bh * M + m] = empty ? -INFINITY : (m_i + cm2) * kLn2 + __logf(l_tot);
   }
 }
+
+// explicit instantiations: every (dtype, head dim) pair the dispatcher can reach
+#define FOX_INSTANTIATE_FWD(TR)                                   \
+  template __global__ void fwd_kernel<TR, 16>(const FwdK);        \
+  template __global__ void fwd_kernel<TR, 32>(const FwdK);        \
+  template __global__ void fwd_kernel<TR, 64>(const FwdK);        \
+  template __global__ void fwd_kernel<TR, 128>(const FwdK);
+FOX_INSTANTIATE_FWD(Bf16)
+FOX_INSTANTIATE_FWD(Fp16)
 
 template <typename Tr>
 static hipError_t launch_fwd_t(const FwdK& a, int D, hipStream_t s) {
