@@ -49,17 +49,73 @@ __global__ __launch_bounds__(256) void delta_kernel(const BwdK a) {
 }
 
 // ---------------------------------------------------------------------------
+// One step (kKvBM query rows) of the dK/dV kernel for one wave (32 key rows).
+template <typename Tr, int D>
+__device__ inline void dkdv_step(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
+                                 const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16], f32x16 (&dkacc)[(D + 31) / 32],
+                                 f32x16 (&dvacc)[(D + 31) / 32], float& csum, int a_s0, int n, int n_w0, float qk_scale,
+                                 float colc, int lane) {
+  constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32;
+  const int g = lane >> 5, i = lane & 31;
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int a_b0 = a_s0 + 32 * mb;   // key position of the block's first query row
+    if (a_b0 + 31 < n_w0) continue;    // block entirely above the diagonal for this wave
+    f32x16 s = Tr::mfma32(lds_row_operand<D>(q_tile, 32 * mb + i, g), kreg[0], zero);
+#pragma unroll
+    for (int kk = 1; kk < KK; ++kk) s = Tr::mfma32(lds_row_operand<D>(q_tile, 32 * mb + i, 2 * kk + g), kreg[kk], s);
+    f32x16 dp = Tr::mfma32(lds_row_operand<D>(do_tile, 32 * mb + i, g), vreg[0], zero);
+#pragma unroll
+    for (int kk = 1; kk < KK; ++kk) dp = Tr::mfma32(lds_row_operand<D>(do_tile, 32 * mb + i, 2 * kk + g), vreg[kk], dp);
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const f32x4 rc = *reinterpret_cast<const f32x4*>(&rc_s[32 * mb + 8 * q4 + 4 * g]);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) s[4 * q4 + t] = __builtin_amdgcn_exp2f(fmaf(s[4 * q4 + t], qk_scale, rc[t]) - colc);
+    }
+    if (a_b0 < n_w0 + 31) {  // causal compare, only on blocks that cross the diagonal
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = (n > a_b0 + c_row(r, g)) ? 0.f : s[r];
+    }
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const f32x4 dl = *reinterpret_cast<const f32x4*>(&dl_s[32 * mb + 8 * q4 + 4 * g]);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const float ds = s[4 * q4 + t] * (dp[4 * q4 + t] - dl[t]);
+        dp[4 * q4 + t] = ds;
+        csum += ds;
+      }
+    }
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const u32x4 pb = pack8<Tr>(s, 8 * hh);
+      const u32x4 dsb = pack8<Tr>(dp, 8 * hh);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        dvacc[db] = Tr::mfma32(lds_col_operand<D>(do_tile, 32 * mb + 16 * hh, db, lane), pb, dvacc[db]);
+        dkacc[db] = Tr::mfma32(lds_col_operand<D>(q_tile, 32 * mb + 16 * hh, db, lane), dsb, dkacc[db]);
+      }
+    }
+  }
+}
+
 template <typename Tr, int D>
 __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
-  constexpr int BN = kKvBN, BMQ = kKvBM, NT = 256;
-  constexpr int KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32;
+  constexpr int BN = kKvBN, BMQ = kKvBM;
+  constexpr int KK = D / 16, DB = (D + 31) / 32;
   static_assert(BN == 128, "four waves of 32 key rows");
-  __shared__ __align__(16) char q_tile[BMQ * D * 2];
-  __shared__ __align__(16) char do_tile[BMQ * D * 2];
-  __shared__ __align__(16) float rc_s[BMQ];
-  __shared__ __align__(16) float dl_s[BMQ];
+  __shared__ __align__(16) char q_tile0[Tile<D>::bytes(BMQ)];
+  __shared__ __align__(16) char q_tile1[Tile<D>::bytes(BMQ)];
+  __shared__ __align__(16) char do_tile0[Tile<D>::bytes(BMQ)];
+  __shared__ __align__(16) char do_tile1[Tile<D>::bytes(BMQ)];
+  __shared__ __align__(16) float rc_s0[BMQ];
+  __shared__ __align__(16) float rc_s1[BMQ];
+  __shared__ __align__(16) float dl_s0[BMQ];
+  __shared__ __align__(16) float dl_s1[BMQ];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, i = lane & 31;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), g = lane >> 5, i = lane & 31;
   int bh, nt;
   decode_block(blockIdx.x, a.n_tiles, a.B * a.H, bh, nt);
   const int b = bh / a.H, h = bh % a.H;
@@ -91,6 +147,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     m_hi = min(M, u * BMQ);
   }
   if (n0 + BN <= seq) m_hi = m_lo;  // every key of the tile is left padding
+  const int n_steps = m_hi > m_lo ? (m_hi - m_lo + BMQ - 1) / BMQ : 0;
 
   const int n_w0 = n0 + 32 * wave;
   const int n = n_w0 + i;  // this lane's key row
@@ -108,73 +165,38 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
   float csum = 0.f;
 
-  TileLoader<D, BMQ, NT> ql, dol;
+  const DirectTileLoader<D, BMQ> qld(a.q.st, wave, lane), dold(a.d_o.st, wave, lane);
   float rc_pref = 0.f, dl_pref = 0.f;
-  auto prefetch = [&](int ms) {
-    ql.load(qp, a.q.st, ms, M, tid);
-    dol.load(dop, a.d_o.st, ms, M, tid);
-    if (tid < BMQ) {
-      const int mm = ms + tid;
-      rc_pref = -INFINITY;
-      dl_pref = 0.f;
-      if (mm < M) {
-        const float l = lse_row[mm];
-        if (l > -INFINITY) rc_pref = (c_row[p_seq + mm] - c_ref - l) * kLog2e;
-        dl_pref = delta_row[mm];
-      }
+  auto issue = [&](int ms, char* qt, char* dot) {
+    if (tid < BMQ) {  // small loads first and branch-free: vmcnt retires in order
+      const int mm = ms + tid, mc = min(mm, M - 1);
+      const float l = lse_row[mc], cv = c_row[p_seq + mc], dv = delta_row[mc];
+      rc_pref = (mm < M && l > -INFINITY) ? (cv - c_ref - l) * kLog2e : -INFINITY;
+      dl_pref = mm < M ? dv : 0.f;
     }
+    qld.issue(qp, a.q.st, ms, M, qt);
+    dold.issue(dop, a.d_o.st, ms, M, dot);
   };
-  if (m_lo < m_hi) prefetch(m_lo);
+  auto compute = [&](int ms, const char* qt, const char* dot, const float* rc, const float* dl) {
+    dkdv_step<Tr, D>(qt, dot, rc, dl, kreg, vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane);
+  };
 
-  for (int ms = m_lo; ms < m_hi; ms += BMQ) {
+  if (n_steps > 0) {
+    issue(m_lo, q_tile0, do_tile0);
+    if (tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
+  }
+  for (int t = 0; t < n_steps; t += 2) {
+    wait_vmem_all();
     __syncthreads();
-    ql.store(q_tile, tid);
-    dol.store(do_tile, tid);
-    if (tid < BMQ) { rc_s[tid] = rc_pref; dl_s[tid] = dl_pref; }
+    if (t + 1 < n_steps) issue(m_lo + (t + 1) * BMQ, q_tile1, do_tile1);
+    compute(m_lo + t * BMQ, q_tile0, do_tile0, rc_s0, dl_s0);
+    if (t + 1 >= n_steps) break;
+    if (tid < BMQ) { rc_s1[tid] = rc_pref; dl_s1[tid] = dl_pref; }
+    wait_vmem_all();
     __syncthreads();
-    if (ms + BMQ < m_hi) prefetch(ms + BMQ);
-
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      const int a_b0 = p_seq + ms + 32 * mb;  // key position of the block's first query row
-      if (a_b0 + 31 < n_w0) continue;         // block entirely above the diagonal for this wave
-      const bool diag = a_b0 < n_w0 + 31;
-      f32x16 s, dp;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) s = Tr::mfma32(lds_row_operand<D>(q_tile, 32 * mb + i, 2 * kk + g), kreg[kk], s);
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) dp = Tr::mfma32(lds_row_operand<D>(do_tile, 32 * mb + i, 2 * kk + g), vreg[kk], dp);
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const f32x4 rc = *reinterpret_cast<const f32x4*>(&rc_s[32 * mb + 8 * q4 + 4 * g]);
-        const f32x4 dl = *reinterpret_cast<const f32x4*>(&dl_s[32 * mb + 8 * q4 + 4 * g]);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int r = 4 * q4 + t;
-          float p = __builtin_amdgcn_exp2f(fmaf(s[r], qk_scale, rc[t]) - colc);
-          if (diag) {
-            const int am = a_b0 + 8 * q4 + 4 * g + t;
-            p = (n > am) ? 0.f : p;
-          }
-          const float ds = p * (dp[r] - dl[t]);
-          s[r] = p;
-          dp[r] = ds;
-          csum += ds;
-        }
-      }
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        const u32x4 pb = pack8<Tr>(s, 8 * hh);
-        const u32x4 dsb = pack8<Tr>(dp, 8 * hh);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          dvacc[db] = Tr::mfma32(lds_col_operand<D>(do_tile, 32 * mb + 16 * hh, db, lane), pb, dvacc[db]);
-          dkacc[db] = Tr::mfma32(lds_col_operand<D>(q_tile, 32 * mb + 16 * hh, db, lane), dsb, dkacc[db]);
-        }
-      }
-    }
+    if (t + 2 < n_steps) issue(m_lo + (t + 2) * BMQ, q_tile0, do_tile0);
+    compute(m_lo + (t + 1) * BMQ, q_tile1, do_tile1, rc_s1, dl_s1);
+    if (t + 2 < n_steps && tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
   }
 
   const float ctot = half_sum(csum);
@@ -199,15 +221,62 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
 }
 
 // ---------------------------------------------------------------------------
+// One 64-key tile of the dQ kernel for one wave (32 query rows).
 template <typename Tr, int D>
-__global__ __launch_bounds__(256) void dq_kernel(const BwdK a) {
-  constexpr int BM = kFwdBM, BN = kFwdBN, NT = 256;
-  constexpr int KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
-  __shared__ __align__(16) char k_tile[BN * D * 2];
-  __shared__ __align__(16) char v_tile[BN * D * 2];
-  __shared__ __align__(16) float cn_s[BN];
+__device__ inline void dq_tile(const char* k_tile, const char* v_tile, const float* cn_s, const u32x4 (&qreg)[D / 16],
+                               const u32x4 (&doreg)[D / 16], f32x16 (&dqacc)[(D + 31) / 32], float& rsum, int n0, int a_m,
+                               int a_w0, float qk_scale, float rowc, float delta, int lane) {
+  constexpr int BN = kFwdBN, KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
+  const int g = lane >> 5, i = lane & 31;
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int nb0 = n0 + 32 * nb;
+    if (nb0 > a_w0 + 31) continue;  // block entirely above this wave's rows
+    f32x16 s = Tr::mfma32(lds_row_operand<D>(k_tile, 32 * nb + i, g), qreg[0], zero);
+#pragma unroll
+    for (int kk = 1; kk < KK; ++kk) s = Tr::mfma32(lds_row_operand<D>(k_tile, 32 * nb + i, 2 * kk + g), qreg[kk], s);
+    f32x16 dp = Tr::mfma32(lds_row_operand<D>(v_tile, 32 * nb + i, g), doreg[0], zero);
+#pragma unroll
+    for (int kk = 1; kk < KK; ++kk) dp = Tr::mfma32(lds_row_operand<D>(v_tile, 32 * nb + i, 2 * kk + g), doreg[kk], dp);
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const f32x4 cn = *reinterpret_cast<const f32x4*>(&cn_s[32 * nb + 8 * q4 + 4 * g]);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) s[4 * q4 + t] = __builtin_amdgcn_exp2f(fmaf(s[4 * q4 + t], qk_scale, rowc) - cn[t]);
+    }
+    if (nb0 + 31 > a_w0) {  // causal compare, only on blocks that cross the diagonal
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = (nb0 + c_row(r, g) > a_m) ? 0.f : s[r];
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float ds = s[r] * (dp[r] - delta);
+      dp[r] = ds;
+      rsum += ds;
+    }
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const u32x4 dsb = pack8<Tr>(dp, 8 * hh);
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        dqacc[db] = Tr::mfma32(lds_col_operand<D>(k_tile, 32 * nb + 16 * hh, db, lane), dsb, dqacc[db]);
+    }
+  }
+}
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, i = lane & 31;
+template <typename Tr, int D>
+__global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
+  constexpr int BM = kFwdBM, BN = kFwdBN;
+  constexpr int KK = D / 16, DB = (D + 31) / 32;
+  __shared__ __align__(16) char k_tile0[Tile<D>::bytes(BN)];
+  __shared__ __align__(16) char k_tile1[Tile<D>::bytes(BN)];
+  __shared__ __align__(16) char v_tile0[Tile<D>::bytes(BN)];
+  __shared__ __align__(16) char v_tile1[Tile<D>::bytes(BN)];
+  __shared__ __align__(16) float cn_s0[BN];
+  __shared__ __align__(16) float cn_s1[BN];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), g = lane >> 5, i = lane & 31;
   int bh, mt;
   decode_block(blockIdx.x, a.n_tiles, a.B * a.H, bh, mt);
   const int b = bh / a.H, h = bh % a.H;
@@ -233,6 +302,7 @@ __global__ __launch_bounds__(256) void dq_kernel(const BwdK a) {
     lo = max(lo, t * BN);
   }
   lo = (lo / BN) * BN;
+  const int n_tiles = (hi - lo + BN - 1) / BN;
 
   const int m = m0 + 32 * wave + i;
   const int a_m = p_seq + m;
@@ -256,62 +326,37 @@ __global__ __launch_bounds__(256) void dq_kernel(const BwdK a) {
     for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
   float rsum = 0.f;
 
-  TileLoader<D, BN, NT> kl, vl;
+  const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
   float cn_pref = 0.f;
-  auto prefetch = [&](int nn0) {
-    kl.load(kp, a.k.st, nn0, N, tid);
-    vl.load(vp, a.v.st, nn0, N, tid);
-    if (tid < BN) {
-      const int nn = nn0 + tid;
-      cn_pref = (nn < N && nn >= seq) ? (c_row[nn] - c_ref) * kLog2e : INFINITY;
+  auto issue = [&](int n0, char* kt, char* vt) {
+    if (tid < BN) {  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
+      const int nn = n0 + tid;
+      const float cv = c_row[min(nn, N - 1)];
+      cn_pref = (nn < N && nn >= seq) ? (cv - c_ref) * kLog2e : INFINITY;
     }
+    kld.issue(kp, a.k.st, n0, N, kt);
+    vld.issue(vp, a.v.st, n0, N, vt);
   };
-  if (lo < hi) prefetch(lo);
+  auto compute = [&](int n0, const char* kt, const char* vt, const float* cn) {
+    dq_tile<Tr, D>(kt, vt, cn, qreg, doreg, dqacc, rsum, n0, a_m, a_w0, qk_scale, rowc, delta, lane);
+  };
 
-  for (int n0 = lo; n0 < hi; n0 += BN) {
+  if (n_tiles > 0) {
+    issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
+    if (tid < BN) cn_s0[tid] = cn_pref;
+  }
+  for (int t = n_tiles - 1; t >= 0; t -= 2) {
+    wait_vmem_all();
     __syncthreads();
-    kl.store(k_tile, tid);
-    vl.store(v_tile, tid);
-    if (tid < BN) cn_s[tid] = cn_pref;
+    if (t >= 1) issue(lo + (t - 1) * BN, k_tile1, v_tile1);
+    compute(lo + t * BN, k_tile0, v_tile0, cn_s0);
+    if (t < 1) break;
+    if (tid < BN) cn_s1[tid] = cn_pref;
+    wait_vmem_all();
     __syncthreads();
-    if (n0 + BN < hi) prefetch(n0 + BN);
-
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      const int nb0 = n0 + 32 * nb;
-      if (nb0 > a_w0 + 31) continue;  // block entirely above this wave's rows
-      const bool diag = nb0 + 31 > a_w0;
-      f32x16 s, dp;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) s = Tr::mfma32(lds_row_operand<D>(k_tile, 32 * nb + i, 2 * kk + g), qreg[kk], s);
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) dp = Tr::mfma32(lds_row_operand<D>(v_tile, 32 * nb + i, 2 * kk + g), doreg[kk], dp);
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const f32x4 cn = *reinterpret_cast<const f32x4*>(&cn_s[32 * nb + 8 * q4 + 4 * g]);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int r = 4 * q4 + t;
-          float p = __builtin_amdgcn_exp2f(fmaf(s[r], qk_scale, rowc) - cn[t]);
-          if (diag) {
-            const int nn = nb0 + 8 * q4 + 4 * g + t;
-            p = (nn > a_m) ? 0.f : p;
-          }
-          const float ds = p * (dp[r] - delta);
-          dp[r] = ds;
-          rsum += ds;
-        }
-      }
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        const u32x4 dsb = pack8<Tr>(dp, 8 * hh);
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-          dqacc[db] = Tr::mfma32(lds_col_operand<D>(k_tile, 32 * nb + 16 * hh, db, lane), dsb, dqacc[db]);
-      }
-    }
+    if (t >= 2) issue(lo + (t - 2) * BN, k_tile0, v_tile0);
+    compute(lo + (t - 1) * BN, k_tile1, v_tile1, cn_s1);
+    if (t >= 2 && tid < BN) cn_s0[tid] = cn_pref;
   }
 
   const float rtot = half_sum(rsum);
@@ -331,6 +376,19 @@ __global__ __launch_bounds__(256) void dq_kernel(const BwdK a) {
     if (g == 0) a.dc[(int64_t)bh * N + a_m] += rtot;  // the dK/dV kernel wrote the column part earlier on this stream
   }
 }
+
+// explicit instantiations: every (dtype, head dim) pair the dispatchers can reach
+#define FOX_INSTANTIATE_BWD(KERNEL, TR)                      \
+  template __global__ void KERNEL<TR, 16>(const BwdK);       \
+  template __global__ void KERNEL<TR, 32>(const BwdK);       \
+  template __global__ void KERNEL<TR, 64>(const BwdK);       \
+  template __global__ void KERNEL<TR, 128>(const BwdK);
+FOX_INSTANTIATE_BWD(delta_kernel, Bf16)
+FOX_INSTANTIATE_BWD(delta_kernel, Fp16)
+FOX_INSTANTIATE_BWD(dkdv_kernel, Bf16)
+FOX_INSTANTIATE_BWD(dkdv_kernel, Fp16)
+FOX_INSTANTIATE_BWD(dq_kernel, Bf16)
+FOX_INSTANTIATE_BWD(dq_kernel, Fp16)
 
 // ---------------------------------------------------------------------------
 #define FOX_DISPATCH_D(KERNEL, GRID, SMEM)                                                        \

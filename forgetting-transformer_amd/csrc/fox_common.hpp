@@ -72,21 +72,28 @@ __device__ inline u32x4 pack8(const f32x16& c, int first) {
 __device__ inline int c_row(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
 
 // ---------------------------------------------------------------------------
-// LDS tile: ROWS x D 16-bit elements, dense rows of D*2 bytes, 16-byte chunks
-// XOR-swizzled by a row-dependent pattern so that both read patterns below
-// spread over all banks.
+// LDS tile of ROWS x D 16-bit elements, organised in blocks of 64 sixteen-byte
+// slots (1 KiB of data = 4 lines of 256 bytes; for D = 128 a line is a row), the
+// unit one LDS-direct load instruction fills.  Blocks are 1040 bytes apart and
+// within a block the slot index inside line l is XORed with 4*l.  With that
+//   * 16 lanes reading the same chunk of 16 consecutive rows (MFMA row operand,
+//     ds_read_b128) hit 16 different bank groups: 4 from the XOR, 4 from the pad;
+//   * 32 lanes reading 4 rows x 64 bytes (transposed operand, ds_read_b64_tr_b16)
+//     cover all 64 banks exactly once;
+//   * the address is  lane term(chunk bits 2-3) + immediate(other chunk bits, row
+//     block), so a kernel keeps 4 address registers per read pattern.
 // ---------------------------------------------------------------------------
 template <int D>
 struct Tile {
-  static constexpr int CH = D / 8;
-  static constexpr int ROW_BYTES = D * 2;
-  static __device__ inline int swz(int row) {
-    if constexpr (CH == 16) return ((row & 3) << 2) | ((row >> 2) & 3);
-    else if constexpr (CH == 8) return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
-    else if constexpr (CH == 4) return (row >> 2) & 3;
-    else return (row >> 3) & 1;
+  static constexpr int CH = D / 8;             // 16-byte chunks per row
+  static constexpr int RPB = 64 / CH;          // rows per block
+  static constexpr int BLOCK_BYTES = 1040;
+  static constexpr int bytes(int rows) { return rows / RPB * BLOCK_BYTES; }
+  static __device__ inline int off(int row, int chunk) {
+    const int p = (row % RPB) * CH + chunk;    // slot within the block
+    const int line = p >> 4, q = p & 15;
+    return (row / RPB) * BLOCK_BYTES + line * 256 + ((q ^ (line << 2)) << 4);
   }
-  static __device__ inline int off(int row, int chunk) { return row * ROW_BYTES + ((chunk ^ swz(row)) << 4); }
 };
 
 // Row operand: eight consecutive elements (one chunk) of one row.
@@ -156,8 +163,8 @@ struct TileLoader {
 // HBM -> LDS tile loader without registers: buffer loads with the LDS bit.  Each
 // wave instruction moves 64 x 16 bytes into a contiguous 1 KiB block of LDS (slot
 // of lane l = block base + 16*l, whatever address the lane reads from), so the
-// swizzle is applied on the global side: the lane that owns LDS slot (row, c')
-// fetches chunk c' ^ swz(row) of that row.  Rows at or beyond row_limit lie
+// swizzle is applied on the global side: each lane fetches the (row, chunk) that
+// the tile layout assigns to its slot.  Rows at or beyond row_limit lie
 // outside the buffer resource and read as zero.  The caller waits for vmcnt(0) and
 // a barrier before the tile is read.
 // ---------------------------------------------------------------------------
@@ -177,9 +184,11 @@ struct DirectTileLoader {
   __device__ inline DirectTileLoader(int64_t row_stride, int wave_, int lane) : wave(wave_) {
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const int pos = (wave + 4 * j) * 64 + lane;
-      const int row = pos / CH, cp = pos % CH;
-      voff[j] = (int)(row * row_stride * 2) + ((cp ^ Tile<D>::swz(row)) << 4);
+      // physical slot of this lane inside block (wave + 4j) -> the (row, chunk) stored there
+      const int line = lane >> 4, q = (lane & 15) ^ (line << 2);
+      const int p = line * 16 + q;
+      const int row = (wave + 4 * j) * Tile<D>::RPB + p / CH, c = p % CH;
+      voff[j] = (int)(row * row_stride * 2) + (c << 4);
     }
   }
   __device__ inline void issue(const uint16_t* base, int64_t row_stride, int row0, int row_limit, char* tile) const {
@@ -190,7 +199,7 @@ struct DirectTileLoader {
     for (int j = 0; j < PER; ++j) {
       const int blk = wave + 4 * j;
       if (NBLK % 4 == 0 || blk < NBLK)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(tile + blk * 1024), 16, voff[j], 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(tile + blk * Tile<D>::BLOCK_BYTES), 16, voff[j], 0, 0, 0);
     }
   }
 };

@@ -119,10 +119,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   constexpr int BM = kFwdBM, BN = kFwdBN;
   constexpr int KK = D / 16, DB = (D + 31) / 32;
   static_assert(BM == 128, "four waves of 32 rows");
-  __shared__ __align__(16) char k_tile0[BN * D * 2];
-  __shared__ __align__(16) char k_tile1[BN * D * 2];
-  __shared__ __align__(16) char v_tile0[BN * D * 2];
-  __shared__ __align__(16) char v_tile1[BN * D * 2];
+  __shared__ __align__(16) char k_tile0[Tile<D>::bytes(BN)];
+  __shared__ __align__(16) char k_tile1[Tile<D>::bytes(BN)];
+  __shared__ __align__(16) char v_tile0[Tile<D>::bytes(BN)];
+  __shared__ __align__(16) char v_tile1[Tile<D>::bytes(BN)];
   __shared__ __align__(16) float cn_s0[BN];
   __shared__ __align__(16) float cn_s1[BN];
 
@@ -173,12 +173,13 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
   float cn_pref = 0.f;
   auto issue = [&](int n0, char* kt, char* vt) {
+    if (tid < BN) {  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
+      const int n = n0 + tid;
+      const float cv = c_row[min(n, N - 1)];
+      cn_pref = (n < N && n >= seq) ? (cv - c_ref) * kLog2e : INFINITY;
+    }
     kld.issue(kp, a.k.st, n0, N, kt);
     vld.issue(vp, a.v.st, n0, N, vt);
-    if (tid < BN) {
-      const int n = n0 + tid;
-      cn_pref = (n < N && n >= seq) ? (c_row[n] - c_ref) * kLog2e : INFINITY;
-    }
   };
   auto compute = [&](int n0, const char* kt, const char* vt, const float* cn) {
     if (n0 > a_w0 + 31) return;  // tile entirely above this wave's rows
