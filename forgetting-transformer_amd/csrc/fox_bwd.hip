@@ -101,6 +101,100 @@ __device__ inline void dkdv_step(const char* q_tile, const char* do_tile, const 
   }
 }
 
+// Interior step (every query row of the step sits at or below every key of the
+// tile: no causal compare, nothing to skip): branch-free and software-pipelined by
+// hand, because the kernel holds one wave per SIMD and nobody else can fill the
+// matrix pipe while this wave does its exp/scale arithmetic.  The step is cut
+// into slots; slot b issues, interleaved in chunks of 4 MFMAs + 2 scores,
+//   * the score MFMAs        S, dP   of block b+1,
+//   * the vector arithmetic  P, dS   of block b,
+//   * the accumulation MFMAs dV, dK  of block b-1,
+// which are mutually independent.  A scheduling fence after every chunk keeps the
+// compiler from regrouping them; LDS operands of the next chunk are requested
+// before the fence so their latency hides behind the current chunk.
+template <typename Tr, int D>
+__device__ inline void dkdv_step_interior(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
+                                          const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16],
+                                          f32x16 (&dkacc)[(D + 31) / 32], f32x16 (&dvacc)[(D + 31) / 32], float& csum,
+                                          float qk_scale, float colc, int lane) {
+  constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32, NCH = 8;
+  static_assert(KK <= NCH && 2 * DB <= NCH, "one k-step and one accumulation pair per chunk");
+  const int g = lane >> 5, i = lane & 31;
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  f32x16 s[MB], dp[MB];
+  u32x4 pb[MB][2], dsb[MB][2];
+#pragma unroll
+  for (int slot = -1; slot <= MB; ++slot) {
+    const bool do_s = slot + 1 < MB, do_v = slot >= 0 && slot < MB, do_c = slot >= 1;
+    const int bs = slot + 1, bv = slot, bc = slot - 1;
+    f32x4 rc[4], dl[4];
+    if (do_v) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        rc[q4] = *reinterpret_cast<const f32x4*>(&rc_s[32 * bv + 8 * q4 + 4 * g]);
+        dl[q4] = *reinterpret_cast<const f32x4*>(&dl_s[32 * bv + 8 * q4 + 4 * g]);
+      }
+    }
+    u32x4 aq[NCH + 1], ado[NCH + 1], cq[NCH + 1], cdo[NCH + 1];
+    auto fetch = [&](int u) {
+      if (do_s && u < KK) {
+        aq[u] = lds_row_operand<D>(q_tile, 32 * bs + i, 2 * u + g);
+        ado[u] = lds_row_operand<D>(do_tile, 32 * bs + i, 2 * u + g);
+      }
+      if (do_c && u < 2 * DB) {
+        cdo[u] = lds_col_operand<D>(do_tile, 32 * bc + 16 * (u / DB), u % DB, lane);
+        cq[u] = lds_col_operand<D>(q_tile, 32 * bc + 16 * (u / DB), u % DB, lane);
+      }
+    };
+    fetch(0);
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) {
+      fetch(u + 1);
+      if (do_s && u < KK) {
+        s[bs] = Tr::mfma32(aq[u], kreg[u], u == 0 ? zero : s[bs]);
+        dp[bs] = Tr::mfma32(ado[u], vreg[u], u == 0 ? zero : dp[bs]);
+      }
+      if (do_c && u < 2 * DB) {
+        dvacc[u % DB] = Tr::mfma32(cdo[u], pb[bc][u / DB], dvacc[u % DB]);
+        dkacc[u % DB] = Tr::mfma32(cq[u], dsb[bc][u / DB], dkacc[u % DB]);
+      }
+      if (do_v) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int r = 2 * u + e, q4 = r >> 2, t = r & 3;
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[bv][r], qk_scale, rc[q4][t]) - colc);
+          const float ds = p * (dp[bv][r] - dl[q4][t]);
+          s[bv][r] = p;
+          dp[bv][r] = ds;
+          csum += ds;
+        }
+        if (u % 4 == 3) {  // eight scores complete: pack one MFMA operand each of P and dS
+          pb[bv][u / 4] = pack8<Tr>(s[bv], 8 * (u / 4));
+          dsb[bv][u / 4] = pack8<Tr>(dp[bv], 8 * (u / 4));
+        }
+      }
+      constexpr int kMfmaMask = 0x008, kValuMask = 0x002, kTransMask = 0x400;
+      const int n_mfma = ((do_s && u < KK) ? 2 : 0) + ((do_c && u < 2 * DB) ? 2 : 0);
+      if (do_v && n_mfma == 4) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kValuMask, 5, 0);
+          __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
+        }
+      } else if (do_v && n_mfma == 2) {
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(kValuMask, 10, 0);
+          __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
 template <typename Tr, int D>
 __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   constexpr int BN = kKvBN, BMQ = kKvBM;
@@ -177,26 +271,37 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     qld.issue(qp, a.q.st, ms, M, qt);
     dold.issue(dop, a.d_o.st, ms, M, dot);
   };
-  auto compute = [&](int ms, const char* qt, const char* dot, const float* rc, const float* dl) {
-    dkdv_step<Tr, D>(qt, dot, rc, dl, kreg, vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane);
-  };
-
-  if (n_steps > 0) {
-    issue(m_lo, q_tile0, do_tile0);
+  // Phase 1: the steps that touch the tile's diagonal (at most BN/BMQ + 1 of them) run one at a
+  // time through buffer 0 with the masking code.  Phase 2: interior steps, double-buffered.
+  int n_diag = 0;
+  while (n_diag < n_steps && p_seq + m_lo + n_diag * BMQ < n0 + BN - 1) ++n_diag;
+  for (int t = 0; t < n_diag; ++t) {
+    const int ms = m_lo + t * BMQ;
+    __syncthreads();  // buffer 0 is free again
+    issue(ms, q_tile0, do_tile0);
     if (tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
-  }
-  for (int t = 0; t < n_steps; t += 2) {
     wait_vmem_all();
     __syncthreads();
-    if (t + 1 < n_steps) issue(m_lo + (t + 1) * BMQ, q_tile1, do_tile1);
-    compute(m_lo + t * BMQ, q_tile0, do_tile0, rc_s0, dl_s0);
-    if (t + 1 >= n_steps) break;
+    dkdv_step<Tr, D>(q_tile0, do_tile0, rc_s0, dl_s0, kreg, vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane);
+  }
+  const int m_int = m_lo + n_diag * BMQ, n_int = n_steps - n_diag;
+  if (n_int > 0) {
+    __syncthreads();
+    issue(m_int, q_tile0, do_tile0);
+    if (tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
+  }
+  for (int t = 0; t < n_int; t += 2) {
+    wait_vmem_all();
+    __syncthreads();
+    if (t + 1 < n_int) issue(m_int + (t + 1) * BMQ, q_tile1, do_tile1);
+    dkdv_step_interior<Tr, D>(q_tile0, do_tile0, rc_s0, dl_s0, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane);
+    if (t + 1 >= n_int) break;
     if (tid < BMQ) { rc_s1[tid] = rc_pref; dl_s1[tid] = dl_pref; }
     wait_vmem_all();
     __syncthreads();
-    if (t + 2 < n_steps) issue(m_lo + (t + 2) * BMQ, q_tile0, do_tile0);
-    compute(m_lo + (t + 1) * BMQ, q_tile1, do_tile1, rc_s1, dl_s1);
-    if (t + 2 < n_steps && tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
+    if (t + 2 < n_int) issue(m_int + (t + 2) * BMQ, q_tile0, do_tile0);
+    dkdv_step_interior<Tr, D>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane);
+    if (t + 2 < n_int && tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
   }
 
   const float ctot = half_sum(csum);

@@ -40,7 +40,7 @@ struct BwdK {
 constexpr int kFwdBM = 128;
 constexpr int kFwdBN = 64;
 constexpr int kKvBN = 128;   // key rows per workgroup in the dK/dV kernel
-constexpr int kKvBM = 64;    // query rows per step in the dK/dV kernel
+constexpr int kKvBM = 128;   // query rows per step in the dK/dV kernel
 
 hipError_t launch_fwd(const FwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_bwd_delta(const BwdK& a, int D, int dtype, hipStream_t s);
