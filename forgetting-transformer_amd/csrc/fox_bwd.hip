@@ -51,7 +51,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const BwdK a) {
 // ---------------------------------------------------------------------------
 // One step (kKvBM query rows) of the dK/dV kernel for one wave (32 key rows).
 template <typename Tr, int D>
-__device__ inline void dkdv_step(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
+__device__ __forceinline__ void dkdv_step(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
                                  const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16], f32x16 (&dkacc)[(D + 31) / 32],
                                  f32x16 (&dvacc)[(D + 31) / 32], float& csum, int a_s0, int n, int n_w0, float qk_scale,
                                  float colc, int lane) {
@@ -113,7 +113,7 @@ __device__ inline void dkdv_step(const char* q_tile, const char* do_tile, const 
 // compiler from regrouping them; LDS operands of the next chunk are requested
 // before the fence so their latency hides behind the current chunk.
 template <typename Tr, int D>
-__device__ inline void dkdv_step_interior(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
+__device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
                                           const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16],
                                           f32x16 (&dkacc)[(D + 31) / 32], f32x16 (&dvacc)[(D + 31) / 32], float& csum,
                                           float qk_scale, float colc, int lane) {
@@ -272,22 +272,23 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     dold.issue(dop, a.d_o.st, ms, M, dot);
   };
   // Phase 1: the steps that touch the tile's diagonal (at most BN/BMQ + 1 of them) run one at a
-  // time through buffer 0 with the masking code.  Phase 2: interior steps, double-buffered.
+  // time through buffer 1 with the masking code; the first interior tile is requested into
+  // buffer 0 before the last of them is computed.  Phase 2: interior steps, double-buffered.
   int n_diag = 0;
   while (n_diag < n_steps && p_seq + m_lo + n_diag * BMQ < n0 + BN - 1) ++n_diag;
+  const int m_int = m_lo + n_diag * BMQ, n_int = n_steps - n_diag;
   for (int t = 0; t < n_diag; ++t) {
     const int ms = m_lo + t * BMQ;
-    __syncthreads();  // buffer 0 is free again
-    issue(ms, q_tile0, do_tile0);
-    if (tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
+    __syncthreads();  // buffer 1 is free again
+    issue(ms, q_tile1, do_tile1);
+    if (tid < BMQ) { rc_s1[tid] = rc_pref; dl_s1[tid] = dl_pref; }
     wait_vmem_all();
     __syncthreads();
-    dkdv_step<Tr, D>(q_tile0, do_tile0, rc_s0, dl_s0, kreg, vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane);
+    if (t == n_diag - 1 && n_int > 0) issue(m_int, q_tile0, do_tile0);
+    dkdv_step<Tr, D>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane);
   }
-  const int m_int = m_lo + n_diag * BMQ, n_int = n_steps - n_diag;
   if (n_int > 0) {
-    __syncthreads();
-    issue(m_int, q_tile0, do_tile0);
+    if (n_diag == 0) issue(m_int, q_tile0, do_tile0);
     if (tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
   }
   for (int t = 0; t < n_int; t += 2) {
@@ -328,7 +329,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
 // ---------------------------------------------------------------------------
 // One 64-key tile of the dQ kernel for one wave (32 query rows).
 template <typename Tr, int D>
-__device__ inline void dq_tile(const char* k_tile, const char* v_tile, const float* cn_s, const u32x4 (&qreg)[D / 16],
+__device__ __forceinline__ void dq_tile(const char* k_tile, const char* v_tile, const float* cn_s, const u32x4 (&qreg)[D / 16],
                                const u32x4 (&doreg)[D / 16], f32x16 (&dqacc)[(D + 31) / 32], float& rsum, int n0, int a_m,
                                int a_w0, float qk_scale, float rowc, float delta, int lane) {
   constexpr int BN = kFwdBN, KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;

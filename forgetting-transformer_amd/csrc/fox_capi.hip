@@ -43,6 +43,13 @@ int check_view(const fox_view* v, const char* name) {
   return FOX_OK;
 }
 
+// The tile loaders address one (batch, head) slice with 32-bit byte offsets.
+int check_extent(const fox_view* v, int rows, int D, const char* name) {
+  const int64_t bytes = ((int64_t)(rows - 1) * v->stride_t + D) * 2;
+  if (v->stride_t <= 0 || bytes >= (int64_t)1 << 31) return fail(FOX_E_ARG, "%s: one (batch, head) slice must span less than 2 GiB with a positive row stride", name);
+  return FOX_OK;
+}
+
 fox::View to_view(const fox_view& v) { return fox::View{(const uint16_t*)v.ptr, v.stride_b, v.stride_h, v.stride_t}; }
 
 #define FOX_TRY(x)            \
@@ -68,6 +75,10 @@ int make_bwd(const fox_bwd_args* args, fox::BwdK& k, bool need_grads) {
   FOX_TRY(check_view(&args->q, "q"));
   FOX_TRY(check_view(&args->k, "k"));
   FOX_TRY(check_view(&args->v, "v"));
+  FOX_TRY(check_extent(&args->q, args->dims.M, args->dims.D, "q"));
+  FOX_TRY(check_extent(&args->d_o, args->dims.M, args->dims.D, "do"));
+  FOX_TRY(check_extent(&args->k, args->dims.N, args->dims.D, "k"));
+  FOX_TRY(check_extent(&args->v, args->dims.N, args->dims.D, "v"));
   if (!args->log_lambda || !args->lse || !args->dlog_lambda) return fail(FOX_E_ARG, "log_lambda, lse and dlog_lambda must not be NULL");
   k.q = to_view(args->q);
   k.k = to_view(args->k);
@@ -122,6 +133,14 @@ int fox_auto_threshold(const fox_dims* dims, const fox_view* q, const fox_view* 
                    "fox_auto_threshold");
 }
 
+int fox_attn_fwd_workspace_bytes(const fox_dims* dims, int64_t* bytes) {
+  FOX_TRY(check_dims(dims));
+  if (!bytes) return fail(FOX_E_ARG, "bytes is NULL");
+  const int splits = fox::fwd_key_splits(dims->B, dims->H, dims->M, dims->N);
+  *bytes = splits <= 1 ? 0 : (int64_t)splits * dims->B * dims->H * dims->M * (dims->D + 2) * (int64_t)sizeof(float);
+  return FOX_OK;
+}
+
 int fox_attn_fwd(const fox_fwd_args* args, void* stream) {
   if (!args) return fail(FOX_E_ARG, "args is NULL");
   FOX_TRY(check_dims(&args->dims));
@@ -129,6 +148,8 @@ int fox_attn_fwd(const fox_fwd_args* args, void* stream) {
   FOX_TRY(check_view(&args->k, "k"));
   FOX_TRY(check_view(&args->v, "v"));
   FOX_TRY(check_view(&args->o, "o"));
+  FOX_TRY(check_extent(&args->k, args->dims.N, args->dims.D, "k"));
+  FOX_TRY(check_extent(&args->v, args->dims.N, args->dims.D, "v"));
   if (!args->log_lambda || !args->lse) return fail(FOX_E_ARG, "log_lambda and lse must not be NULL");
   fox::FwdK k{};
   k.q = to_view(args->q);
@@ -143,6 +164,18 @@ int fox_attn_fwd(const fox_fwd_args* args, void* stream) {
   k.B = args->dims.B; k.H = args->dims.H; k.M = args->dims.M; k.N = args->dims.N;
   k.sm_scale = args->sm_scale;
   k.n_mtiles = (args->dims.M + fox::kFwdBM - 1) / fox::kFwdBM;
+  k.splits = 1;
+  if (args->workspace) {
+    int64_t need = 0;
+    FOX_TRY(fox_attn_fwd_workspace_bytes(&args->dims, &need));
+    if (need > 0) {
+      if (args->workspace_bytes < need) return fail(FOX_E_ARG, "workspace too small: %lld < %lld bytes", (long long)args->workspace_bytes, (long long)need);
+      if (((uintptr_t)args->workspace & 15) != 0) return fail(FOX_E_ALIGN, "workspace must be 16-byte aligned");
+      k.splits = fox::fwd_key_splits(k.B, k.H, k.M, k.N);
+      k.ws_o = (float*)args->workspace;
+      k.ws_ml = k.ws_o + (int64_t)k.splits * k.B * k.H * k.M * args->dims.D;
+    }
+  }
   return check_hip(fox::launch_fwd(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), "fox_attn_fwd");
 }
 

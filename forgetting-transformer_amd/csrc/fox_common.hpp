@@ -27,32 +27,32 @@ constexpr int kWave = 64;
 // fp32 <-> 16-bit conversions differ.
 // ---------------------------------------------------------------------------
 struct Bf16 {
-  static __device__ inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+  static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
-  static __device__ inline uint32_t pack2(float lo, float hi) {
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     bf16x2 v = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(uint32_t, v);
   }
-  static __device__ inline float lo(uint32_t w) { return __uint_as_float(w << 16); }
-  static __device__ inline float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+  static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 };
 
 struct Fp16 {
-  static __device__ inline f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+  static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
-  static __device__ inline uint32_t pack2(float lo, float hi) {
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     f16x2 v = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(uint32_t, v);
   }
-  static __device__ inline float lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
-  static __device__ inline float hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
+  static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
+  static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
 };
 
 // Pack eight consecutive accumulator values into one 16-byte MFMA operand.
 template <typename Tr>
-__device__ inline u32x4 pack8(const f32x16& c, int first) {
+__device__ __forceinline__ u32x4 pack8(const f32x16& c, int first) {
   u32x4 r;
   r[0] = Tr::pack2(c[first + 0], c[first + 1]);
   r[1] = Tr::pack2(c[first + 2], c[first + 3]);
@@ -69,7 +69,7 @@ __device__ inline u32x4 pack8(const f32x16& c, int first) {
 // contraction index: operand element e = 4*u + t of k-slice h (16 rows) is
 // accumulator register r = 8*h + e, i.e. C row 16*h + 8*u + 4*g + t.
 // ---------------------------------------------------------------------------
-__device__ inline int c_row(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+__device__ __forceinline__ int c_row(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
 
 // ---------------------------------------------------------------------------
 // LDS tile of ROWS x D 16-bit elements, organised in blocks of 64 sixteen-byte
@@ -89,7 +89,7 @@ struct Tile {
   static constexpr int RPB = 64 / CH;          // rows per block
   static constexpr int BLOCK_BYTES = 1040;
   static constexpr int bytes(int rows) { return rows / RPB * BLOCK_BYTES; }
-  static __device__ inline int off(int row, int chunk) {
+  static __device__ __forceinline__ int off(int row, int chunk) {
     const int p = (row % RPB) * CH + chunk;    // slot within the block
     const int line = p >> 4, q = p & 15;
     return (row / RPB) * BLOCK_BYTES + line * 256 + ((q ^ (line << 2)) << 4);
@@ -98,11 +98,11 @@ struct Tile {
 
 // Row operand: eight consecutive elements (one chunk) of one row.
 template <int D>
-__device__ inline u32x4 lds_row_operand(const char* tile, int row, int chunk) {
+__device__ __forceinline__ u32x4 lds_row_operand(const char* tile, int row, int chunk) {
   return *reinterpret_cast<const u32x4*>(tile + Tile<D>::off(row, chunk));
 }
 
-__device__ inline u32x2 lds_tr_read(const char* p) {
+__device__ __forceinline__ u32x2 lds_tr_read(const char* p) {
   typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
   s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
   return __builtin_bit_cast(u32x2, v);
@@ -114,7 +114,7 @@ __device__ inline u32x2 lds_tr_read(const char* p) {
 // 16 lanes: lane x of a block supplies the address of 4 consecutive columns
 // 4*(x%4).. of row (x/4), and receives column x of those four rows.
 template <int D>
-__device__ inline u32x4 lds_col_operand(const char* tile, int row16, int db, int lane) {
+__device__ __forceinline__ u32x4 lds_col_operand(const char* tile, int row16, int db, int lane) {
   const int g = lane >> 5, blk = (lane >> 4) & 1, x = lane & 15;
   int col = 32 * db + 16 * blk + 4 * (x & 3);
   if constexpr (D < 32) col &= (D - 1);  // columns >= D feed output rows nobody stores
@@ -138,7 +138,7 @@ struct TileLoader {
   static constexpr int PER = (CHUNKS + NT - 1) / NT;
   u32x4 reg[PER];
 
-  __device__ inline void load(const uint16_t* base, int64_t row_stride, int row0, int row_limit, int tid) {
+  __device__ __forceinline__ void load(const uint16_t* base, int64_t row_stride, int row0, int row_limit, int tid) {
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const int idx = tid + j * NT;
@@ -149,7 +149,7 @@ struct TileLoader {
         reg[j] = *reinterpret_cast<const u32x4*>(base + (int64_t)(row0 + row) * row_stride + ch * 8);
     }
   }
-  __device__ inline void store(char* tile, int tid) const {
+  __device__ __forceinline__ void store(char* tile, int tid) const {
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const int idx = tid + j * NT;
@@ -170,7 +170,7 @@ struct TileLoader {
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
-__device__ inline void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), other counters untouched
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), other counters untouched
 
 template <int D, int ROWS>
 struct DirectTileLoader {
@@ -181,7 +181,7 @@ struct DirectTileLoader {
   int voff[PER];
   int wave;
 
-  __device__ inline DirectTileLoader(int64_t row_stride, int wave_, int lane) : wave(wave_) {
+  __device__ __forceinline__ DirectTileLoader(int64_t row_stride, int wave_, int lane) : wave(wave_) {
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       // physical slot of this lane inside block (wave + 4j) -> the (row, chunk) stored there
@@ -191,7 +191,7 @@ struct DirectTileLoader {
       voff[j] = (int)(row * row_stride * 2) + (c << 4);
     }
   }
-  __device__ inline void issue(const uint16_t* base, int64_t row_stride, int row0, int row_limit, char* tile) const {
+  __device__ __forceinline__ void issue(const uint16_t* base, int64_t row_stride, int row0, int row_limit, char* tile) const {
     const uint16_t* p = base + (int64_t)row0 * row_stride;
     const int64_t bytes = row_limit > row0 ? ((int64_t)(row_limit - 1 - row0) * row_stride + D) * 2 : 0;
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, (int)bytes, 0x00020000);
@@ -207,7 +207,7 @@ struct DirectTileLoader {
 // Operand held in registers for a whole kernel: lane (g, i) keeps row (row0 + i),
 // elements 16*kk + 8*g .. +7 for every k-step kk.  Rows >= row_limit are zero.
 template <int D>
-__device__ inline void load_row_operand_regs(u32x4 (&dst)[D / 16], const uint16_t* base, int64_t row_stride, int row,
+__device__ __forceinline__ void load_row_operand_regs(u32x4 (&dst)[D / 16], const uint16_t* base, int64_t row_stride, int row,
                                              int row_limit, int g) {
 #pragma unroll
   for (int kk = 0; kk < D / 16; ++kk) {
@@ -221,12 +221,12 @@ __device__ inline void load_row_operand_regs(u32x4 (&dst)[D / 16], const uint16_
 // Wave helpers
 // ---------------------------------------------------------------------------
 // Value held by the partner lane in the other 32-lane half.
-__device__ inline float half_max(float x) {
+__device__ __forceinline__ float half_max(float x) {
   unsigned v = __float_as_uint(x);
   auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
-__device__ inline float half_sum(float x) {
+__device__ __forceinline__ float half_sum(float x) {
   unsigned v = __float_as_uint(x);
   auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
@@ -235,7 +235,7 @@ __device__ inline float half_sum(float x) {
 // Workgroup id -> (bh, tile) with every tile of one (batch, head) on one XCD (the
 // hardware deals consecutive workgroup ids round-robin over 8 XCDs, each with its
 // own L2), heaviest tiles (largest index under a causal mask) first.
-__device__ inline void decode_block(int wid, int n_tiles, int n_bh, int& bh, int& tile) {
+__device__ __forceinline__ void decode_block(int wid, int n_tiles, int n_bh, int& bh, int& tile) {
   if ((n_bh & 7) == 0) {
     const int xcd = wid & 7, seq = wid >> 3;
     bh = (seq / n_tiles) * 8 + xcd;
@@ -250,7 +250,7 @@ __device__ inline void decode_block(int wid, int n_tiles, int n_bh, int& bh, int
 // in [0, t_max] whose largest decay  c_out - c[last column of the block]  is not
 // below thr.  c is non-increasing, so the blocks before it are exactly the
 // prunable ones.  Evaluated by all 64 lanes at once; the result is wave-uniform.
-__device__ inline int acp_first_kept_block(const float* c_row, float c_out, float thr, int N, int BN, int t_max, int lane) {
+__device__ __forceinline__ int acp_first_kept_block(const float* c_row, float c_out, float thr, int N, int BN, int t_max, int lane) {
   for (int base = 0; base <= t_max; base += kWave) {
     const int t = base + lane;
     bool keep = false;
@@ -268,7 +268,7 @@ __device__ inline int acp_first_kept_block(const float* c_row, float c_out, floa
 // Key-side bound: the first query block (BMQ rows, first row u*BMQ) in [u_lo, U)
 // whose largest decay against the key tile,  c[P_SEQ + u*BMQ] - c_last,  is below
 // thr; every later block is prunable too.  Returns U when none is.
-__device__ inline int acp_first_pruned_qblock(const float* c_row, float c_last, float thr, int p_seq, int BMQ, int u_lo,
+__device__ __forceinline__ int acp_first_pruned_qblock(const float* c_row, float c_last, float thr, int p_seq, int BMQ, int u_lo,
                                               int U, int lane) {
   for (int base = u_lo; base < U; base += kWave) {
     const int u = base + lane;

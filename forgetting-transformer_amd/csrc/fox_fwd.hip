@@ -33,7 +33,7 @@ namespace fox {
 constexpr float kLazyMaxLog2 = 8.0f;
 
 template <typename Tr, int D>
-__device__ inline void fwd_tile(const char* k_tile, const char* v_tile, const float* cn_s, const u32x4 (&qreg)[D / 16],
+__device__ __forceinline__ void fwd_tile(const char* k_tile, const char* v_tile, const float* cn_s, const u32x4 (&qreg)[D / 16],
                                 f32x16 (&oacc)[(D + 31) / 32], float& m_i, float& l_i, int n0, int a_m, float qk_scale,
                                 int lane, bool diag) {
   constexpr int BN = kFwdBN, KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
@@ -114,7 +114,7 @@ __device__ inline void fwd_tile(const char* k_tile, const char* v_tile, const fl
   }
 }
 
-template <typename Tr, int D>
+template <typename Tr, int D, bool SPLIT>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   constexpr int BM = kFwdBM, BN = kFwdBN;
   constexpr int KK = D / 16, DB = (D + 31) / 32;
@@ -127,8 +127,15 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   __shared__ __align__(16) float cn_s1[BN];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), g = lane >> 5, i = lane & 31;
-  int bh, mt;
-  decode_block(blockIdx.x, a.n_mtiles, a.B * a.H, bh, mt);
+  int bh, mt, sp = 0;
+  if constexpr (SPLIT) {  // (query tile, key split) pairs take the place of query tiles
+    int mts;
+    decode_block(blockIdx.x, a.n_mtiles * a.splits, a.B * a.H, bh, mts);
+    mt = mts / a.splits;
+    sp = mts % a.splits;
+  } else {
+    decode_block(blockIdx.x, a.n_mtiles, a.B * a.H, bh, mt);
+  }
   const int b = bh / a.H, h = bh % a.H;
   const int M = a.M, N = a.N, p_seq = N - M;
   const int m0 = mt * BM;
@@ -151,8 +158,14 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     lo = max(lo, t * BN);
   }
   lo = (lo / BN) * BN;
-  if (a.first_block && tid == 0) a.first_block[(int64_t)bh * a.n_mtiles + mt] = lo / BN;
-  const int n_tiles = (hi - lo + BN - 1) / BN;  // walked from the last (diagonal) tile down to lo
+  if (a.first_block && tid == 0 && sp == 0) a.first_block[(int64_t)bh * a.n_mtiles + mt] = lo / BN;
+  int n_tiles = (hi - lo + BN - 1) / BN;  // walked from the last (diagonal) tile down to lo
+  if constexpr (SPLIT) {  // this workgroup's contiguous share of the key tiles
+    const int per = (n_tiles + a.splits - 1) / a.splits;
+    const int t0 = min(n_tiles, sp * per), t1 = min(n_tiles, t0 + per);
+    lo += t0 * BN;
+    n_tiles = t1 - t0;
+  }
 
   const int m = m0 + 32 * wave + i;  // this lane's query row
   const int a_m = p_seq + m;
@@ -208,6 +221,29 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
 
   // epilogue
   const float l_tot = half_sum(l_i);
+  if constexpr (SPLIT) {
+    // partial result of this key split: unnormalised accumulator, row maximum (log2 domain,
+    // including the row term) and row sum; fox::combine_kernel merges the splits
+    if (m < M) {
+      const int64_t row = ((int64_t)sp * a.B * a.H + bh) * M + m;
+      float* wo = a.ws_o + row * D;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int d = 32 * db + 8 * q4 + 4 * g;
+          if (d < D) {
+            f32x4 w = {oacc[db][4 * q4 + 0], oacc[db][4 * q4 + 1], oacc[db][4 * q4 + 2], oacc[db][4 * q4 + 3]};
+            *reinterpret_cast<f32x4*>(wo + d) = w;
+          }
+        }
+      if (g == 0) {
+        a.ws_ml[2 * row] = m_i + cm2;
+        a.ws_ml[2 * row + 1] = l_tot;
+      }
+    }
+    return;
+  }
   const bool empty = a_m < seq;
   const float inv = empty ? 0.f : 1.0f / l_tot;
   if (m < M) {
@@ -227,30 +263,98 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   }
 }
 
+// Merge the partial results of the key splits of one query row:
+//   m = max_s m_s,  l = sum_s l_s 2^(m_s - m),  o = sum_s acc_s 2^(m_s - m) / l,  lse = m ln2 + ln l.
+// One thread per (row, 4 head-dim elements).
+template <typename Tr, int D>
+__global__ __launch_bounds__(256) void combine_kernel(const FwdK a) {
+  constexpr int TPR = D / 4;  // threads per row
+  const int64_t n_rows = (int64_t)a.B * a.H * a.M;
+  const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / TPR;
+  const int d = (threadIdx.x % TPR) * 4;
+  if (row >= n_rows) return;
+  const int bh = (int)(row / a.M), m = (int)(row % a.M), b = bh / a.H, h = bh % a.H;
+  float mx = -INFINITY;
+  for (int sp = 0; sp < a.splits; ++sp) mx = fmaxf(mx, a.ws_ml[2 * (sp * n_rows + row)]);
+  float l = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int sp = 0; sp < a.splits; ++sp) {
+    const int64_t r = sp * n_rows + row;
+    const float w = __builtin_amdgcn_exp2f(a.ws_ml[2 * r] - mx);
+    l += a.ws_ml[2 * r + 1] * w;
+    const f32x4 o = *reinterpret_cast<const f32x4*>(a.ws_o + r * D + d);
+    acc += o * w;
+  }
+  int seq = 0;
+  if (a.seq_start) {
+    const int64_t s64 = a.seq_start[b];
+    seq = (int)(s64 < 0 ? 0 : (s64 > a.N ? a.N : s64));
+  }
+  const bool empty = (a.N - a.M + m) < seq;
+  const float inv = empty ? 0.f : 1.0f / l;
+  uint16_t* op = const_cast<uint16_t*>(a.o.ptr) + b * a.o.sb + h * a.o.sh + (int64_t)m * a.o.st + d;
+  u32x2 w;
+  w[0] = Tr::pack2(acc[0] * inv, acc[1] * inv);
+  w[1] = Tr::pack2(acc[2] * inv, acc[3] * inv);
+  *reinterpret_cast<u32x2*>(op) = w;
+  if (d == 0) a.lse[row] = empty ? -INFINITY : mx * kLn2 + __logf(l);
+}
+
 // explicit instantiations: every (dtype, head dim) pair the dispatcher can reach
-#define FOX_INSTANTIATE_FWD(TR)                                   \
-  template __global__ void fwd_kernel<TR, 16>(const FwdK);        \
-  template __global__ void fwd_kernel<TR, 32>(const FwdK);        \
-  template __global__ void fwd_kernel<TR, 64>(const FwdK);        \
-  template __global__ void fwd_kernel<TR, 128>(const FwdK);
+#define FOX_INSTANTIATE_FWD(TR)                                          \
+  template __global__ void fwd_kernel<TR, 16, false>(const FwdK);        \
+  template __global__ void fwd_kernel<TR, 32, false>(const FwdK);        \
+  template __global__ void fwd_kernel<TR, 64, false>(const FwdK);        \
+  template __global__ void fwd_kernel<TR, 128, false>(const FwdK);       \
+  template __global__ void fwd_kernel<TR, 16, true>(const FwdK);         \
+  template __global__ void fwd_kernel<TR, 32, true>(const FwdK);         \
+  template __global__ void fwd_kernel<TR, 64, true>(const FwdK);         \
+  template __global__ void fwd_kernel<TR, 128, true>(const FwdK);        \
+  template __global__ void combine_kernel<TR, 16>(const FwdK);           \
+  template __global__ void combine_kernel<TR, 32>(const FwdK);           \
+  template __global__ void combine_kernel<TR, 64>(const FwdK);           \
+  template __global__ void combine_kernel<TR, 128>(const FwdK);
 FOX_INSTANTIATE_FWD(Bf16)
 FOX_INSTANTIATE_FWD(Fp16)
 
+template <typename Tr, int D>
+static hipError_t launch_fwd_d(const FwdK& a, hipStream_t s) {
+  if (a.splits <= 1) {
+    hipLaunchKernelGGL((fwd_kernel<Tr, D, false>), dim3((unsigned)(a.n_mtiles * a.B * a.H)), dim3(256), 0, s, a);
+    return hipGetLastError();
+  }
+  hipLaunchKernelGGL((fwd_kernel<Tr, D, true>), dim3((unsigned)(a.n_mtiles * a.splits * a.B * a.H)), dim3(256), 0, s, a);
+  const int64_t threads = (int64_t)a.B * a.H * a.M * (D / 4);
+  hipLaunchKernelGGL((combine_kernel<Tr, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, a);
+  return hipGetLastError();
+}
+
 template <typename Tr>
 static hipError_t launch_fwd_t(const FwdK& a, int D, hipStream_t s) {
-  const dim3 grid((unsigned)(a.n_mtiles * a.B * a.H)), block(256);
   switch (D) {
-    case 16: hipLaunchKernelGGL((fwd_kernel<Tr, 16>), grid, block, 0, s, a); break;
-    case 32: hipLaunchKernelGGL((fwd_kernel<Tr, 32>), grid, block, 0, s, a); break;
-    case 64: hipLaunchKernelGGL((fwd_kernel<Tr, 64>), grid, block, 0, s, a); break;
-    case 128: hipLaunchKernelGGL((fwd_kernel<Tr, 128>), grid, block, 0, s, a); break;
+    case 16: return launch_fwd_d<Tr, 16>(a, s);
+    case 32: return launch_fwd_d<Tr, 32>(a, s);
+    case 64: return launch_fwd_d<Tr, 64>(a, s);
+    case 128: return launch_fwd_d<Tr, 128>(a, s);
     default: return hipErrorInvalidValue;
   }
-  return hipGetLastError();
 }
 
 hipError_t launch_fwd(const FwdK& a, int D, int dtype, hipStream_t s) {
   return dtype == 0 ? launch_fwd_t<Bf16>(a, D, s) : launch_fwd_t<Fp16>(a, D, s);
+}
+
+// Number of key splits the forward uses for a shape: 1 unless the grid of query tiles
+// alone leaves most of the chip idle while each workgroup has a long key loop (chunked
+// prefill, decode).  Splits are sized to give every CU about two workgroups.
+int fwd_key_splits(int B, int H, int M, int N) {
+  const int64_t wgs = (int64_t)((M + kFwdBM - 1) / kFwdBM) * B * H;
+  const int key_tiles = (N + kFwdBN - 1) / kFwdBN;
+  if (wgs >= 512 || key_tiles < 16) return 1;
+  int splits = (int)((512 + wgs - 1) / wgs);
+  splits = splits > key_tiles / 8 ? key_tiles / 8 : splits;
+  splits = splits > 32 ? 32 : splits;
+  return splits < 1 ? 1 : splits;
 }
 
 }  // namespace fox

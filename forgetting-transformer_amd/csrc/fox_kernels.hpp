@@ -21,6 +21,9 @@ struct FwdK {
   int B, H, M, N;
   float sm_scale;
   int n_mtiles;
+  int splits;      // key splits of the forward (1 = none)
+  float* ws_o;     // (splits, B, H, M, D) partial accumulators
+  float* ws_ml;    // (splits, B, H, M, 2) partial row maximum and row sum
 };
 
 struct BwdK {
@@ -43,6 +46,7 @@ constexpr int kKvBN = 128;   // key rows per workgroup in the dK/dV kernel
 constexpr int kKvBM = 128;   // query rows per step in the dK/dV kernel
 
 hipError_t launch_fwd(const FwdK& a, int D, int dtype, hipStream_t s);
+int fwd_key_splits(int B, int H, int M, int N);
 hipError_t launch_bwd_delta(const BwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_bwd_dkdv(const BwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_bwd_dq(const BwdK& a, int D, int dtype, hipStream_t s);

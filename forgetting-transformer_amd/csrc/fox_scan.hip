@@ -85,7 +85,7 @@ hipError_t launch_cumsum_bwd(const float* dc, float* dg, int B, int H, int N, hi
 // "auto" threshold
 // ---------------------------------------------------------------------------
 template <typename Tr>
-__device__ inline float round16(float x) {  // round to the 16-bit dtype and back
+__device__ __forceinline__ float round16(float x) {  // round to the 16-bit dtype and back
   return Tr::lo(Tr::pack2(x, 0.f));
 }
 

@@ -142,10 +142,14 @@ class ForgettingAttention(torch.autograd.Function):
             if return_start_index:
                 block_m, _, _, _ = _lib.tile_config(D)
                 first_block = torch.zeros((B, H, (M + block_m - 1) // block_m), dtype=torch.int32, device=device)
+            ws_bytes = C.c_int64(0)
+            _lib.check(lib.fox_attn_fwd_workspace_bytes(C.byref(dims), C.byref(ws_bytes)), "fox_attn_fwd_workspace_bytes")
+            workspace = torch.empty(ws_bytes.value, dtype=torch.uint8, device=device) if ws_bytes.value > 0 else None
             args = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), log_lambda.data_ptr(), L.data_ptr(),
                                 None if seq_start is None else seq_start.data_ptr(),
                                 None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
-                                sm_scale, None if first_block is None else first_block.data_ptr())
+                                sm_scale, None if first_block is None else first_block.data_ptr(),
+                                None if workspace is None else workspace.data_ptr(), ws_bytes.value)
             _lib.check(lib.fox_attn_fwd(C.byref(args), stream), "fox_attn_fwd")
 
         ctx.save_for_backward(q, k, v, o, L, log_lambda, seq_start, adaptive_threshold)

@@ -88,6 +88,8 @@ typedef struct fox_fwd_args {
   const float* threshold;     /* (B,H) contiguous or NULL (no pruning) */
   float sm_scale;
   int32_t* first_block;       /* optional (B,H,ceil(M/block_m)): first key block each query block visits */
+  void* workspace;            /* optional scratch of fox_attn_fwd_workspace_bytes() bytes, 16-byte aligned; NULL = never split keys */
+  int64_t workspace_bytes;    /* size of workspace; too small a workspace is an error */
 } fox_fwd_args;
 
 /*
@@ -96,6 +98,16 @@ typedef struct fox_fwd_args {
  * by ForgettingAttention.forward (:159-204).
  */
 int fox_attn_fwd(const fox_fwd_args* args, void* stream);
+
+/*
+ * Scratch the forward can use to split the key loop of each query tile over several
+ * workgroups (flash-decoding style partial (max, sum, accumulator) + combine).  Shapes with
+ * few query tiles and long key sequences -- chunked prefill, decode (the reference's
+ * M == 1 path, :148-153) -- otherwise leave most of the chip idle.  *bytes is 0 when the
+ * shape is not split.  No counterpart in the reference, which always runs one program per
+ * query tile (:186).
+ */
+int fox_attn_fwd_workspace_bytes(const fox_dims* dims, int64_t* bytes);
 
 typedef struct fox_bwd_args {
   fox_dims dims;

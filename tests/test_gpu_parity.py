@@ -151,6 +151,20 @@ def test_aggressive_threshold_prunes_exactly_the_reported_tiles(fa, thr):
         assert torch.isfinite(x).all()
 
 
+@pytest.mark.parametrize("B,H,M,N,D,seq,thr", [(1, 2, 1, 8192, 64, None, None), (2, 2, 128, 4096, 128, [100, 3000], None),
+                                                (1, 3, 200, 6000, 64, None, -10.0), (2, 1, 1, 2000, 128, [0, 1999], None),
+                                                (1, 1, 64, 9000, 32, [8990], "auto"), (1, 2, 300, 5000, 16, None, None)])
+def test_key_split_shapes(fa, B, H, M, N, D, seq, thr):
+    """Few query tiles and a long key sequence (decode, chunked prefill): the forward splits the
+    key loop over several workgroups and merges the partial results."""
+    import ctypes as C_
+    from forgetting_transformer.ops import _lib
+    need = C_.c_int64(0)
+    _lib.check(_lib.load().fox_attn_fwd_workspace_bytes(C_.byref(_lib.Dims(B, H, M, N, D, 0)), C_.byref(need)), "ws")
+    assert need.value > 0, "this shape is meant to exercise the split path"
+    run_case(fa, B, H, M, N, D, seq_start=seq, thr=thr, seed=N, gate_mean=4.0, gate_std=1.0)
+
+
 @pytest.mark.parametrize("sm_scale", [None, 0.5, 1.3])
 def test_sm_scale(fa, sm_scale):
     run_case(fa, 1, 2, 260, 260, 64, sm_scale=sm_scale, qkv_std=0.5, seed=3)

@@ -59,6 +59,18 @@ def test_c_abi_rejects_bad_arguments_before_launching():
         _lib.check(-1, "x")
 
 
+def test_workspace_query():
+    lib = _lib.load()
+    need = C.c_int64(-1)
+    assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(4, 16, 16384, 16384, 128, 0)), C.byref(need)) == 0
+    assert need.value == 0                          # plenty of query tiles: never split
+    assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(16, 16, 128, 32768, 128, 0)), C.byref(need)) == 0
+    assert need.value > 0 and need.value % (16 * 16 * 128 * 130 * 4) == 0   # splits x rows x (D + 2) floats
+    assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(1, 1, 1, 100, 64, 0)), C.byref(need)) == 0 and need.value == 0
+    assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(1, 1, 1, 100, 48, 0)), C.byref(need)) == -1
+    assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(1, 1, 1, 100, 64, 0)), None) == -1
+
+
 def _cpu_inputs(B=2, T=8, H=2, D=64, dtype=torch.bfloat16):
     q = torch.randn(B, T, H, D).to(dtype)
     g = torch.nn.functional.logsigmoid(torch.randn(B, T, H))
