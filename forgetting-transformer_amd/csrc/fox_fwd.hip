@@ -114,10 +114,108 @@ __device__ __forceinline__ void fwd_tile(const char* k_tile, const char* v_tile,
   }
 }
 
+// Interior tile (no key of the tile is right of any query row of the workgroup): branch-free and
+// software-pipelined across tiles.  While the vector ALU turns the scores of the current tile into
+// probabilities, the matrix pipe already computes the scores of the next tile (from k_next) and then
+// accumulates the current tile's P V (from v_cur).  s_cur holds the raw scores of the current tile
+// on entry; s_next holds those of the next tile on exit.  Work is issued in small chunks separated
+// by scheduling fences so that MFMA and vector instructions alternate in the instruction stream.
+template <typename Tr, int D>
+__device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const char* v_cur, const float* cn_s,
+                                                  const u32x4 (&qreg)[D / 16], f32x16 (&oacc)[(D + 31) / 32], float& m_i,
+                                                  float& l_i, float qk_scale, int lane, f32x16 (&s_cur)[kFwdBN / 32],
+                                                  f32x16 (&s_next)[kFwdBN / 32]) {
+  constexpr int BN = kFwdBN, KK = D / 16, DB = (D + 31) / 32, NB = BN / 32, NSL = BN / 16;
+  constexpr int SPC = 16 * NB / KK;  // scores handled per chunk of phase A
+  static_assert(16 * NB % KK == 0 && SPC % 4 == 0, "whole float4 groups of scores per chunk");
+  const int g = lane >> 5, i = lane & 31;
+  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  // Phase A: scores of the next tile  ||  x = s*scale - cn and the running maximum of the current tile
+  float mloc = -INFINITY;
+  u32x4 ka[NB][KK + 1];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) ka[nb][0] = lds_row_operand<D>(k_next, 32 * nb + i, g);
+#pragma unroll
+  for (int u = 0; u < KK; ++u) {
+    if (u + 1 < KK) {
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) ka[nb][u + 1] = lds_row_operand<D>(k_next, 32 * nb + i, 2 * (u + 1) + g);
+    }
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) s_next[nb] = Tr::mfma32(ka[nb][u], qreg[u], u == 0 ? zero : s_next[nb]);
+#pragma unroll
+    for (int e4 = 0; e4 < SPC / 4; ++e4) {
+      const int first = u * SPC + 4 * e4, nb = first >> 4, q4 = (first & 15) >> 2;
+      const f32x4 cn = *reinterpret_cast<const f32x4*>(&cn_s[32 * nb + 8 * q4 + 4 * g]);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const float x = fmaf(s_cur[nb][4 * q4 + t], qk_scale, -cn[t]);
+        s_cur[nb][4 * q4 + t] = x;
+        mloc = fmaxf(mloc, x);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  mloc = half_max(mloc);
+  const bool raise = mloc > m_i + kLazyMaxLog2;
+  if (__any(raise)) {  // rare: rescale what has been accumulated so far
+    const float m_new = raise ? mloc : m_i;
+    const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+    m_i = m_new;
+    l_i *= alpha;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+  }
+
+  // Phase B: p = exp2(x - m), row sums, pack  ||  O^T += V^T P^T, one 16-key slice behind
+  float rsum = 0.f;
+  u32x4 pb[NSL];
+  u32x4 va[NSL][DB];
+#pragma unroll
+  for (int c = 0; c <= NSL; ++c) {
+    if (c < NSL) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) va[c][db] = lds_col_operand<D>(v_cur, 16 * c, db, lane);
+    }
+    if (c >= 1) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) oacc[db] = Tr::mfma32(va[c - 1][db], pb[c - 1], oacc[db]);
+    }
+    if (c < NSL) {
+      const int nb = c >> 1, r0 = 8 * (c & 1);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __builtin_amdgcn_exp2f(s_cur[nb][r0 + e] - m_i);
+        s_cur[nb][r0 + e] = p;
+        rsum += p;
+      }
+      pb[c] = pack8<Tr>(s_cur[nb], r0);
+    }
+    if (c >= 1 && c < NSL) {
+#pragma unroll
+      for (int k = 0; k < DB; ++k) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  l_i += rsum;
+}
+
 template <typename Tr, int D, bool SPLIT>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   constexpr int BM = kFwdBM, BN = kFwdBN;
-  constexpr int KK = D / 16, DB = (D + 31) / 32;
+  constexpr int KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
   static_assert(BM == 128, "four waves of 32 rows");
   __shared__ __align__(16) char k_tile0[Tile<D>::bytes(BN)];
   __shared__ __align__(16) char k_tile1[Tile<D>::bytes(BN)];
@@ -199,24 +297,78 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     fwd_tile<Tr, D>(kt, vt, cn, qreg, oacc, m_i, l_i, n0, a_m, qk_scale, lane, n0 + BN - 1 > a_w0);
   };
 
-  if (n_tiles > 0) {
+  // Phase 1: the tiles that reach the workgroup's diagonal (the last ceil(BM/BN) + 1 at most), with
+  // the masking code, double-buffered.  Phase 2: interior tiles, software-pipelined across tiles.
+  int n_diag = 0;
+  while (n_diag < n_tiles && lo + (n_tiles - 1 - n_diag) * BN + BN - 1 > a0) ++n_diag;
+  const int t_stop = n_tiles - n_diag;
+  if (n_diag > 0) {
     issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
     if (tid < BN) cn_s0[tid] = cn_pref;
   }
-  for (int t = n_tiles - 1; t >= 0; t -= 2) {
+  for (int t = n_tiles - 1; t >= t_stop; t -= 2) {
     // even step: consume buffers 0, fill buffers 1
     wait_vmem_all();
     __syncthreads();
-    if (t >= 1) issue(lo + (t - 1) * BN, k_tile1, v_tile1);
+    if (t - 1 >= t_stop) issue(lo + (t - 1) * BN, k_tile1, v_tile1);
     compute(lo + t * BN, k_tile0, v_tile0, cn_s0);
-    if (t < 1) break;
+    if (t - 1 < t_stop) break;
     if (tid < BN) cn_s1[tid] = cn_pref;
     // odd step: consume buffers 1, fill buffers 0
     wait_vmem_all();
     __syncthreads();
-    if (t >= 2) issue(lo + (t - 2) * BN, k_tile0, v_tile0);
+    if (t - 2 >= t_stop) issue(lo + (t - 2) * BN, k_tile0, v_tile0);
     compute(lo + (t - 1) * BN, k_tile1, v_tile1, cn_s1);
-    if (t >= 2 && tid < BN) cn_s0[tid] = cn_pref;
+    if (t - 2 >= t_stop && tid < BN) cn_s0[tid] = cn_pref;
+  }
+
+  const int n_int = t_stop;  // interior tile j (0 = nearest to the diagonal) starts at key lo + (n_int-1-j)*BN
+  if (n_int > 0) {
+    auto issue_k = [&](int j, char* kt) {
+      const int n0 = lo + (n_int - 1 - j) * BN;
+      if (tid < BN) {
+        const int n = n0 + tid;
+        const float cv = c_row[min(n, N - 1)];
+        cn_pref = (n < N && n >= seq) ? (cv - c_ref) * kLog2e : INFINITY;
+      }
+      kld.issue(kp, a.k.st, n0, N, kt);
+    };
+    auto issue_v = [&](int j, char* vt) { vld.issue(vp, a.v.st, lo + (n_int - 1 - j) * BN, N, vt); };
+    // K runs one tile ahead of V: iteration j computes S(j+1) and P(j) V(j).
+    __syncthreads();  // phase 1 is done with every buffer
+    issue_k(0, k_tile0);
+    if (tid < BN) cn_s0[tid] = cn_pref;
+    wait_vmem_all();
+    __syncthreads();
+    if (n_int > 1) issue_k(1, k_tile1);
+    issue_v(0, v_tile0);
+    f32x16 s_a[NB], s_b[NB];
+    {
+      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        s_a[nb] = Tr::mfma32(lds_row_operand<D>(k_tile0, 32 * nb + i, g), qreg[0], zero);
+#pragma unroll
+        for (int kk = 1; kk < KK; ++kk) s_a[nb] = Tr::mfma32(lds_row_operand<D>(k_tile0, 32 * nb + i, 2 * kk + g), qreg[kk], s_a[nb]);
+      }
+    }
+    for (int j = 0; j < n_int; j += 2) {
+      // even iteration: K(j+1) in k_tile1, V(j) in v_tile0, cn(j) in cn_s0
+      wait_vmem_all();
+      __syncthreads();
+      if (j + 1 < n_int && tid < BN) cn_s1[tid] = cn_pref;
+      if (j + 2 < n_int) issue_k(j + 2, k_tile0);
+      if (j + 1 < n_int) issue_v(j + 1, v_tile1);
+      fwd_tile_pipelined<Tr, D>(k_tile1, v_tile0, cn_s0, qreg, oacc, m_i, l_i, qk_scale, lane, s_a, s_b);
+      if (j + 1 >= n_int) break;
+      // odd iteration: K(j+2) in k_tile0, V(j+1) in v_tile1, cn(j+1) in cn_s1
+      wait_vmem_all();
+      __syncthreads();
+      if (j + 2 < n_int && tid < BN) cn_s0[tid] = cn_pref;
+      if (j + 3 < n_int) issue_k(j + 3, k_tile1);
+      if (j + 2 < n_int) issue_v(j + 2, v_tile0);
+      fwd_tile_pipelined<Tr, D>(k_tile0, v_tile1, cn_s1, qreg, oacc, m_i, l_i, qk_scale, lane, s_b, s_a);
+    }
   }
 
   // epilogue
