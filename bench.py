@@ -250,6 +250,8 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extras", action="store_true", help="skip the ACP and chunked-prefill reports")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy three times (a kernel of known traffic to scale HBM counters by)")
     ns = ap.parse_args()
     if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: Forgetting Attention never communicates (every (batch, head) pair is an "
@@ -258,6 +260,14 @@ def main():
         sys.exit("bench.py needs an AMD GPU (there is no CPU path for the operator)")
 
     from forgetting_transformer import forgetting_attention
+
+    if ns.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     w = WORKLOADS[ns.workload]
     tensors = synth(w, "cuda")

@@ -212,6 +212,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), g = lane >> 5, i = lane & 31;
   int bh, nt;
   decode_block(blockIdx.x, a.n_tiles, a.B * a.H, bh, nt);
+  nt = a.n_tiles - 1 - nt;  // the first key tiles see the most query rows: start them first
   const int b = bh / a.H, h = bh % a.H;
   const int M = a.M, N = a.N, p_seq = N - M;
   const int n0 = nt * BN;
@@ -273,10 +274,13 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   };
   // Phase 1: the steps that touch the tile's diagonal (at most BN/BMQ + 1 of them) run one at a
   // time through buffer 1 with the masking code; the first interior tile is requested into
-  // buffer 0 before the last of them is computed.  Phase 2: interior steps, double-buffered.
+  // buffer 0 before the last of them is computed.  Phase 2: interior steps, double-buffered,
+  // from the end of the sequence down: the workgroups of one (batch, head) that run together on
+  // an XCD then request the same Q / dO tile at about the same time, and all but the first
+  // request hit that XCD's L2.
   int n_diag = 0;
   while (n_diag < n_steps && p_seq + m_lo + n_diag * BMQ < n0 + BN - 1) ++n_diag;
-  const int m_int = m_lo + n_diag * BMQ, n_int = n_steps - n_diag;
+  const int n_int = n_steps - n_diag, m_top = m_lo + (n_steps - 1) * BMQ;
   for (int t = 0; t < n_diag; ++t) {
     const int ms = m_lo + t * BMQ;
     __syncthreads();  // buffer 1 is free again
@@ -284,23 +288,23 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     if (tid < BMQ) { rc_s1[tid] = rc_pref; dl_s1[tid] = dl_pref; }
     wait_vmem_all();
     __syncthreads();
-    if (t == n_diag - 1 && n_int > 0) issue(m_int, q_tile0, do_tile0);
+    if (t == n_diag - 1 && n_int > 0) issue(m_top, q_tile0, do_tile0);
     dkdv_step<Tr, D>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane);
   }
   if (n_int > 0) {
-    if (n_diag == 0) issue(m_int, q_tile0, do_tile0);
+    if (n_diag == 0) issue(m_top, q_tile0, do_tile0);
     if (tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
   }
   for (int t = 0; t < n_int; t += 2) {
     wait_vmem_all();
     __syncthreads();
-    if (t + 1 < n_int) issue(m_int + (t + 1) * BMQ, q_tile1, do_tile1);
+    if (t + 1 < n_int) issue(m_top - (t + 1) * BMQ, q_tile1, do_tile1);
     dkdv_step_interior<Tr, D>(q_tile0, do_tile0, rc_s0, dl_s0, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane);
     if (t + 1 >= n_int) break;
     if (tid < BMQ) { rc_s1[tid] = rc_pref; dl_s1[tid] = dl_pref; }
     wait_vmem_all();
     __syncthreads();
-    if (t + 2 < n_int) issue(m_int + (t + 2) * BMQ, q_tile0, do_tile0);
+    if (t + 2 < n_int) issue(m_top - (t + 2) * BMQ, q_tile0, do_tile0);
     dkdv_step_interior<Tr, D>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane);
     if (t + 2 < n_int && tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
   }
