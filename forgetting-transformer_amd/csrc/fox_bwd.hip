@@ -50,6 +50,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const BwdK a) {
 
 // ---------------------------------------------------------------------------
 // One step (kKvBM query rows) of the dK/dV kernel for one wave (32 key rows).
+// rc_s holds rowc_i / (sm_scale*log2e) and dl_s holds -delta_i.
 template <typename Tr, int D>
 __device__ __forceinline__ void dkdv_step(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
                                  const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16], f32x16 (&dkacc)[(D + 31) / 32],
@@ -57,36 +58,26 @@ __device__ __forceinline__ void dkdv_step(const char* q_tile, const char* do_til
                                  float colc, int lane) {
   constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32;
   const int g = lane >> 5, i = lane & 31;
-  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int a_b0 = a_s0 + 32 * mb;   // key position of the block's first query row
     if (a_b0 + 31 < n_w0) continue;    // block entirely above the diagonal for this wave
-    f32x16 s = Tr::mfma32(lds_row_operand<D>(q_tile, 32 * mb + i, g), kreg[0], zero);
+    f32x16 s = acc_init(rc_s, 32 * mb, g), dp = acc_init(dl_s, 32 * mb, g);
 #pragma unroll
-    for (int kk = 1; kk < KK; ++kk) s = Tr::mfma32(lds_row_operand<D>(q_tile, 32 * mb + i, 2 * kk + g), kreg[kk], s);
-    f32x16 dp = Tr::mfma32(lds_row_operand<D>(do_tile, 32 * mb + i, g), vreg[0], zero);
+    for (int kk = 0; kk < KK; ++kk) s = Tr::mfma32(lds_row_operand<D>(q_tile, 32 * mb + i, 2 * kk + g), kreg[kk], s);
 #pragma unroll
-    for (int kk = 1; kk < KK; ++kk) dp = Tr::mfma32(lds_row_operand<D>(do_tile, 32 * mb + i, 2 * kk + g), vreg[kk], dp);
+    for (int kk = 0; kk < KK; ++kk) dp = Tr::mfma32(lds_row_operand<D>(do_tile, 32 * mb + i, 2 * kk + g), vreg[kk], dp);
 #pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      const f32x4 rc = *reinterpret_cast<const f32x4*>(&rc_s[32 * mb + 8 * q4 + 4 * g]);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) s[4 * q4 + t] = __builtin_amdgcn_exp2f(fmaf(s[4 * q4 + t], qk_scale, rc[t]) - colc);
-    }
+    for (int r = 0; r < 16; ++r) s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], qk_scale, -colc));
     if (a_b0 < n_w0 + 31) {  // causal compare, only on blocks that cross the diagonal
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[r] = (n > a_b0 + c_row(r, g)) ? 0.f : s[r];
     }
 #pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      const f32x4 dl = *reinterpret_cast<const f32x4*>(&dl_s[32 * mb + 8 * q4 + 4 * g]);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const float ds = s[4 * q4 + t] * (dp[4 * q4 + t] - dl[t]);
-        dp[4 * q4 + t] = ds;
-        csum += ds;
-      }
+    for (int r = 0; r < 16; ++r) {
+      const float ds = s[r] * dp[r];
+      dp[r] = ds;
+      csum += ds;
     }
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
@@ -120,20 +111,15 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
   constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32, NCH = 8;
   static_assert(KK <= NCH && 2 * DB <= NCH, "one k-step and one accumulation pair per chunk");
   const int g = lane >> 5, i = lane & 31;
-  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   f32x16 s[MB], dp[MB];
   u32x4 pb[MB][2], dsb[MB][2];
 #pragma unroll
   for (int slot = -1; slot <= MB; ++slot) {
     const bool do_s = slot + 1 < MB, do_v = slot >= 0 && slot < MB, do_c = slot >= 1;
     const int bs = slot + 1, bv = slot, bc = slot - 1;
-    f32x4 rc[4], dl[4];
-    if (do_v) {
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        rc[q4] = *reinterpret_cast<const f32x4*>(&rc_s[32 * bv + 8 * q4 + 4 * g]);
-        dl[q4] = *reinterpret_cast<const f32x4*>(&dl_s[32 * bv + 8 * q4 + 4 * g]);
-      }
+    if (do_s) {  // the accumulators start from the row terms instead of zero
+      s[bs] = acc_init(rc_s, 32 * bs, g);
+      dp[bs] = acc_init(dl_s, 32 * bs, g);
     }
     u32x4 aq[NCH + 1], ado[NCH + 1], cq[NCH + 1], cdo[NCH + 1];
     auto fetch = [&](int u) {
@@ -151,8 +137,8 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
     for (int u = 0; u < NCH; ++u) {
       fetch(u + 1);
       if (do_s && u < KK) {
-        s[bs] = Tr::mfma32(aq[u], kreg[u], u == 0 ? zero : s[bs]);
-        dp[bs] = Tr::mfma32(ado[u], vreg[u], u == 0 ? zero : dp[bs]);
+        s[bs] = Tr::mfma32(aq[u], kreg[u], s[bs]);
+        dp[bs] = Tr::mfma32(ado[u], vreg[u], dp[bs]);
       }
       if (do_c && u < 2 * DB) {
         dvacc[u % DB] = Tr::mfma32(cdo[u], pb[bc][u / DB], dvacc[u % DB]);
@@ -161,9 +147,9 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
       if (do_v) {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          const int r = 2 * u + e, q4 = r >> 2, t = r & 3;
-          const float p = __builtin_amdgcn_exp2f(fmaf(s[bv][r], qk_scale, rc[q4][t]) - colc);
-          const float ds = p * (dp[bv][r] - dl[q4][t]);
+          const int r = 2 * u + e;
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[bv][r], qk_scale, -colc));
+          const float ds = p * dp[bv][r];
           s[bv][r] = p;
           dp[bv][r] = ds;
           csum += ds;
@@ -179,14 +165,14 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(kValuMask, 5, 0);
+          __builtin_amdgcn_sched_group_barrier(kValuMask, 4, 0);
           __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
         }
       } else if (do_v && n_mfma == 2) {
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
           __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(kValuMask, 10, 0);
+          __builtin_amdgcn_sched_group_barrier(kValuMask, 8, 0);
           __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
         }
       }
@@ -251,7 +237,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   load_row_operand_regs<D>(vreg, vp, a.v.st, n, N, g);
   const float c_ref = c_row[n0];
   const float colc = (n < N && n >= seq) ? (c_row[n] - c_ref) * kLog2e : INFINITY;
-  const float qk_scale = a.sm_scale * kLog2e;
+  const float qk_scale = nonzero_scale(a.sm_scale * kLog2e), inv_scale = 1.0f / qk_scale;
 
   f32x16 dkacc[DB], dvacc[DB];
 #pragma unroll
@@ -266,8 +252,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     if (tid < BMQ) {  // small loads first and branch-free: vmcnt retires in order
       const int mm = ms + tid, mc = min(mm, M - 1);
       const float l = lse_row[mc], cv = c_row[p_seq + mc], dv = delta_row[mc];
-      rc_pref = (mm < M && l > -INFINITY) ? (cv - c_ref - l) * kLog2e : -INFINITY;
-      dl_pref = mm < M ? dv : 0.f;
+      rc_pref = (mm < M && l > -INFINITY) ? (cv - c_ref - l) * kLog2e * inv_scale : -INFINITY * inv_scale;
+      dl_pref = mm < M ? -dv : 0.f;
     }
     qld.issue(qp, a.q.st, ms, M, qt);
     dold.issue(dop, a.d_o.st, ms, M, dot);
@@ -332,6 +318,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
 
 // ---------------------------------------------------------------------------
 // One 64-key tile of the dQ kernel for one wave (32 query rows).
+// cn_s holds -colc_j / (sm_scale*log2e), the start value of the score accumulators.
 template <typename Tr, int D>
 __device__ __forceinline__ void dq_tile(const char* k_tile, const char* v_tile, const float* cn_s, const u32x4 (&qreg)[D / 16],
                                const u32x4 (&doreg)[D / 16], f32x16 (&dqacc)[(D + 31) / 32], float& rsum, int n0, int a_m,
@@ -343,18 +330,14 @@ __device__ __forceinline__ void dq_tile(const char* k_tile, const char* v_tile, 
   for (int nb = 0; nb < NB; ++nb) {
     const int nb0 = n0 + 32 * nb;
     if (nb0 > a_w0 + 31) continue;  // block entirely above this wave's rows
-    f32x16 s = Tr::mfma32(lds_row_operand<D>(k_tile, 32 * nb + i, g), qreg[0], zero);
+    f32x16 s = acc_init(cn_s, 32 * nb, g);
 #pragma unroll
-    for (int kk = 1; kk < KK; ++kk) s = Tr::mfma32(lds_row_operand<D>(k_tile, 32 * nb + i, 2 * kk + g), qreg[kk], s);
+    for (int kk = 0; kk < KK; ++kk) s = Tr::mfma32(lds_row_operand<D>(k_tile, 32 * nb + i, 2 * kk + g), qreg[kk], s);
     f32x16 dp = Tr::mfma32(lds_row_operand<D>(v_tile, 32 * nb + i, g), doreg[0], zero);
 #pragma unroll
     for (int kk = 1; kk < KK; ++kk) dp = Tr::mfma32(lds_row_operand<D>(v_tile, 32 * nb + i, 2 * kk + g), doreg[kk], dp);
 #pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      const f32x4 cn = *reinterpret_cast<const f32x4*>(&cn_s[32 * nb + 8 * q4 + 4 * g]);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) s[4 * q4 + t] = __builtin_amdgcn_exp2f(fmaf(s[4 * q4 + t], qk_scale, rowc) - cn[t]);
-    }
+    for (int r = 0; r < 16; ++r) s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], qk_scale, rowc));
     if (nb0 + 31 > a_w0) {  // causal compare, only on blocks that cross the diagonal
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[r] = (nb0 + c_row(r, g) > a_m) ? 0.f : s[r];
@@ -427,7 +410,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     if (l > -INFINITY) rowc = (c_row[a_m] - c_ref - l) * kLog2e;
     delta = a.delta[(int64_t)bh * M + m];
   }
-  const float qk_scale = a.sm_scale * kLog2e;
+  const float qk_scale = nonzero_scale(a.sm_scale * kLog2e), inv_scale = 1.0f / qk_scale;
 
   f32x16 dqacc[DB];
 #pragma unroll
@@ -442,7 +425,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     if (tid < BN) {  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
       const int nn = n0 + tid;
       const float cv = c_row[min(nn, N - 1)];
-      cn_pref = (nn < N && nn >= seq) ? (cv - c_ref) * kLog2e : INFINITY;
+      cn_pref = (nn < N && nn >= seq) ? (c_ref - cv) * kLog2e * inv_scale : -INFINITY * inv_scale;
     }
     kld.issue(kp, a.k.st, n0, N, kt);
     vld.issue(vp, a.v.st, n0, N, vt);

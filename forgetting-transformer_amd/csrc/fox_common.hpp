@@ -232,6 +232,26 @@ __device__ __forceinline__ float half_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Start value of a 32x32 MFMA accumulator whose row r carries the per-row term
+// t[row0 + r] (read from LDS): the matrix pipe then adds the dot products to it for
+// free, which saves one vector instruction per score.
+__device__ __forceinline__ f32x16 acc_init(const float* t, int row0, int g) {
+  f32x16 v;
+#pragma unroll
+  for (int q4 = 0; q4 < 4; ++q4) {
+    const f32x4 x = *reinterpret_cast<const f32x4*>(&t[row0 + 8 * q4 + 4 * g]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[4 * q4 + e] = x[e];
+  }
+  return v;
+}
+
+// The kernels fold per-row bias terms into the MFMA accumulators as bias / scale and multiply
+// the finished dot product by scale, so scale must not be zero: a scale below 1e-30 in
+// magnitude is replaced by 1e-30, for which scale * (q.k) still rounds to nothing against
+// the bias.
+__device__ __forceinline__ float nonzero_scale(float s) { return fabsf(s) < 1e-30f ? 1e-30f : s; }
+
 // Workgroup id -> (bh, tile) with every tile of one (batch, head) on one XCD (the
 // hardware deals consecutive workgroup ids round-robin over 8 XCDs, each with its
 // own L2), heaviest tiles (largest index under a causal mask) first.

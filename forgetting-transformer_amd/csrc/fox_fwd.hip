@@ -38,34 +38,25 @@ __device__ __forceinline__ void fwd_tile(const char* k_tile, const char* v_tile,
                                 int lane, bool diag) {
   constexpr int BN = kFwdBN, KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
   const int g = lane >> 5, i = lane & 31;
-  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  // S^T = K Q^T
+  // S^T = K Q^T + key term
   f32x16 s[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     u32x4 ka[KK];
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) ka[kk] = lds_row_operand<D>(k_tile, 32 * nb + i, 2 * kk + g);
-    s[nb] = Tr::mfma32(ka[0], qreg[0], zero);
+    s[nb] = acc_init(cn_s, 32 * nb, g);
 #pragma unroll
-    for (int kk = 1; kk < KK; ++kk) s[nb] = Tr::mfma32(ka[kk], qreg[kk], s[nb]);
+    for (int kk = 0; kk < KK; ++kk) s[nb] = Tr::mfma32(ka[kk], qreg[kk], s[nb]);
   }
 
   // scores in the log2 domain and their maximum
   float mloc = -INFINITY;
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
+  for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4) {
-      const f32x4 cn = *reinterpret_cast<const f32x4*>(&cn_s[32 * nb + 8 * q4 + 4 * g]);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int r = 4 * q4 + t;
-        s[nb][r] = fmaf(s[nb][r], qk_scale, -cn[t]);
-      }
-    }
-  }
+    for (int r = 0; r < 16; ++r) s[nb][r] *= qk_scale;
   if (diag) {  // causal compare, only on tiles that cross the diagonal
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
@@ -121,7 +112,7 @@ __device__ __forceinline__ void fwd_tile(const char* k_tile, const char* v_tile,
 // on entry; s_next holds those of the next tile on exit.  Work is issued in small chunks separated
 // by scheduling fences so that MFMA and vector instructions alternate in the instruction stream.
 template <typename Tr, int D>
-__device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const char* v_cur, const float* cn_s,
+__device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const char* v_cur, const float* cn_next,
                                                   const u32x4 (&qreg)[D / 16], f32x16 (&oacc)[(D + 31) / 32], float& m_i,
                                                   float& l_i, float qk_scale, int lane, f32x16 (&s_cur)[kFwdBN / 32],
                                                   f32x16 (&s_next)[kFwdBN / 32]) {
@@ -129,13 +120,15 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
   constexpr int SPC = 16 * NB / KK;  // scores handled per chunk of phase A
   static_assert(16 * NB % KK == 0 && SPC % 4 == 0, "whole float4 groups of scores per chunk");
   const int g = lane >> 5, i = lane & 31;
-  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  // Phase A: scores of the next tile  ||  x = s*scale - cn and the running maximum of the current tile
+  // Phase A: scores of the next tile  ||  maximum of the current tile's raw scores (sm_scale > 0 here)
   float mloc = -INFINITY;
   u32x4 ka[NB][KK + 1];
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) ka[nb][0] = lds_row_operand<D>(k_next, 32 * nb + i, g);
+  for (int nb = 0; nb < NB; ++nb) {
+    ka[nb][0] = lds_row_operand<D>(k_next, 32 * nb + i, g);
+    s_next[nb] = acc_init(cn_next, 32 * nb, g);
+  }
 #pragma unroll
   for (int u = 0; u < KK; ++u) {
     if (u + 1 < KK) {
@@ -143,26 +136,20 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
       for (int nb = 0; nb < NB; ++nb) ka[nb][u + 1] = lds_row_operand<D>(k_next, 32 * nb + i, 2 * (u + 1) + g);
     }
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) s_next[nb] = Tr::mfma32(ka[nb][u], qreg[u], u == 0 ? zero : s_next[nb]);
+    for (int nb = 0; nb < NB; ++nb) s_next[nb] = Tr::mfma32(ka[nb][u], qreg[u], s_next[nb]);
 #pragma unroll
-    for (int e4 = 0; e4 < SPC / 4; ++e4) {
-      const int first = u * SPC + 4 * e4, nb = first >> 4, q4 = (first & 15) >> 2;
-      const f32x4 cn = *reinterpret_cast<const f32x4*>(&cn_s[32 * nb + 8 * q4 + 4 * g]);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const float x = fmaf(s_cur[nb][4 * q4 + t], qk_scale, -cn[t]);
-        s_cur[nb][4 * q4 + t] = x;
-        mloc = fmaxf(mloc, x);
-      }
+    for (int e = 0; e < SPC; ++e) {
+      const int idx = u * SPC + e;
+      mloc = fmaxf(mloc, s_cur[idx >> 4][idx & 15]);
     }
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
-  mloc = half_max(mloc);
+  mloc = half_max(mloc) * qk_scale;
   const bool raise = mloc > m_i + kLazyMaxLog2;
   if (__any(raise)) {  // rare: rescale what has been accumulated so far
     const float m_new = raise ? mloc : m_i;
@@ -175,7 +162,8 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
       for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
   }
 
-  // Phase B: p = exp2(x - m), row sums, pack  ||  O^T += V^T P^T, one 16-key slice behind
+  // Phase B: p = exp2(s*scale - m), row sums, pack  ||  O^T += V^T P^T, one 16-key slice behind
+  const float neg_m = -m_i;
   float rsum = 0.f;
   u32x4 pb[NSL];
   u32x4 va[NSL][DB];
@@ -193,7 +181,7 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
       const int nb = c >> 1, r0 = 8 * (c & 1);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = __builtin_amdgcn_exp2f(s_cur[nb][r0 + e] - m_i);
+        const float p = __builtin_amdgcn_exp2f(fmaf(s_cur[nb][r0 + e], qk_scale, neg_m));
         s_cur[nb][r0 + e] = p;
         rsum += p;
       }
@@ -272,7 +260,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   load_row_operand_regs<D>(qreg, qp, a.q.st, m, M, g);
   const float c_ref = c_row[a0];
   const float cm2 = (m < M) ? (c_row[a_m] - c_ref) * kLog2e : 0.f;
-  const float qk_scale = a.sm_scale * kLog2e;
+  const float qk_scale = nonzero_scale(a.sm_scale * kLog2e), inv_scale = 1.0f / qk_scale;
 
   f32x16 oacc[DB];
 #pragma unroll
@@ -287,7 +275,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     if (tid < BN) {  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
       const int n = n0 + tid;
       const float cv = c_row[min(n, N - 1)];
-      cn_pref = (n < N && n >= seq) ? (cv - c_ref) * kLog2e : INFINITY;
+      cn_pref = (n < N && n >= seq) ? (c_ref - cv) * kLog2e * inv_scale : -INFINITY * inv_scale;
     }
     kld.issue(kp, a.k.st, n0, N, kt);
     vld.issue(vp, a.v.st, n0, N, vt);
@@ -299,8 +287,11 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
 
   // Phase 1: the tiles that reach the workgroup's diagonal (the last ceil(BM/BN) + 1 at most), with
   // the masking code, double-buffered.  Phase 2: interior tiles, software-pipelined across tiles.
+  // The pipelined code takes the row maximum on the raw accumulators, which needs sm_scale > 0;
+  // otherwise every tile goes through phase 1.
   int n_diag = 0;
   while (n_diag < n_tiles && lo + (n_tiles - 1 - n_diag) * BN + BN - 1 > a0) ++n_diag;
+  if (!(qk_scale > 0.f)) n_diag = n_tiles;
   const int t_stop = n_tiles - n_diag;
   if (n_diag > 0) {
     issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
@@ -329,7 +320,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
       if (tid < BN) {
         const int n = n0 + tid;
         const float cv = c_row[min(n, N - 1)];
-        cn_pref = (n < N && n >= seq) ? (cv - c_ref) * kLog2e : INFINITY;
+        cn_pref = (n < N && n >= seq) ? (c_ref - cv) * kLog2e * inv_scale : -INFINITY * inv_scale;
       }
       kld.issue(kp, a.k.st, n0, N, kt);
     };
@@ -343,31 +334,29 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     if (n_int > 1) issue_k(1, k_tile1);
     issue_v(0, v_tile0);
     f32x16 s_a[NB], s_b[NB];
-    {
-      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        s_a[nb] = Tr::mfma32(lds_row_operand<D>(k_tile0, 32 * nb + i, g), qreg[0], zero);
+    for (int nb = 0; nb < NB; ++nb) {
+      s_a[nb] = acc_init(cn_s0, 32 * nb, g);
 #pragma unroll
-        for (int kk = 1; kk < KK; ++kk) s_a[nb] = Tr::mfma32(lds_row_operand<D>(k_tile0, 32 * nb + i, 2 * kk + g), qreg[kk], s_a[nb]);
-      }
+      for (int kk = 0; kk < KK; ++kk) s_a[nb] = Tr::mfma32(lds_row_operand<D>(k_tile0, 32 * nb + i, 2 * kk + g), qreg[kk], s_a[nb]);
     }
     for (int j = 0; j < n_int; j += 2) {
-      // even iteration: K(j+1) in k_tile1, V(j) in v_tile0, cn(j) in cn_s0
+      // even iteration: K(j+1) in k_tile1 with its key terms in cn_s1, V(j) in v_tile0.  The key
+      // terms of tile j+1 go to LDS before the barrier: their buffer was last read two iterations ago.
       wait_vmem_all();
-      __syncthreads();
       if (j + 1 < n_int && tid < BN) cn_s1[tid] = cn_pref;
+      __syncthreads();
       if (j + 2 < n_int) issue_k(j + 2, k_tile0);
       if (j + 1 < n_int) issue_v(j + 1, v_tile1);
-      fwd_tile_pipelined<Tr, D>(k_tile1, v_tile0, cn_s0, qreg, oacc, m_i, l_i, qk_scale, lane, s_a, s_b);
+      fwd_tile_pipelined<Tr, D>(k_tile1, v_tile0, cn_s1, qreg, oacc, m_i, l_i, qk_scale, lane, s_a, s_b);
       if (j + 1 >= n_int) break;
-      // odd iteration: K(j+2) in k_tile0, V(j+1) in v_tile1, cn(j+1) in cn_s1
+      // odd iteration: K(j+2) in k_tile0 with its key terms in cn_s0, V(j+1) in v_tile1
       wait_vmem_all();
-      __syncthreads();
       if (j + 2 < n_int && tid < BN) cn_s0[tid] = cn_pref;
+      __syncthreads();
       if (j + 3 < n_int) issue_k(j + 3, k_tile1);
       if (j + 2 < n_int) issue_v(j + 2, v_tile0);
-      fwd_tile_pipelined<Tr, D>(k_tile0, v_tile1, cn_s1, qreg, oacc, m_i, l_i, qk_scale, lane, s_b, s_a);
+      fwd_tile_pipelined<Tr, D>(k_tile0, v_tile1, cn_s0, qreg, oacc, m_i, l_i, qk_scale, lane, s_b, s_a);
     }
   }
 

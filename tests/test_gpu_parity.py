@@ -170,6 +170,14 @@ def test_sm_scale(fa, sm_scale):
     run_case(fa, 1, 2, 260, 260, 64, sm_scale=sm_scale, qkv_std=0.5, seed=3)
 
 
+@pytest.mark.parametrize("sm_scale", [0.0, -0.4, 1e-20])
+@pytest.mark.parametrize("M,N", [(400, 400), (130, 700)])
+def test_degenerate_sm_scale(fa, sm_scale, M, N):
+    """Zero, negative and vanishing scales: the kernels carry the decay terms in the MFMA accumulators
+    as term / scale, which must not break down when the scale is not a positive normal number."""
+    run_case(fa, 1, 2, M, N, 64, sm_scale=sm_scale, qkv_std=0.5, seed=5, seq_start=[37])
+
+
 def test_fox_layer_views(fa):
     """The FoX layer passes (B,H,T,D) views of (B,T,H*D) memory and a (B,H,T) view of
     (B,T,H) gates with head_first=True (modeling_forgetting_transformer.py:318-346)."""
