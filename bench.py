@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Forgetting Attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode] [--no-extras] [--no-cpu-baseline]
 
 A step is one forward + backward pass of ``forgetting_attention`` over one batch
 of synthetic input already resident in HBM (forward only for c5).  The default
@@ -39,12 +39,20 @@ import torch  # noqa: E402
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0
 
+# HBM bytes per launch of the dominant kernel of a workload (fetched + written), from two rocprofv3 --pmc
+# passes over this script (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
+# plain 1 GiB copies of --copy-calibration (fetch x2.00, write x1.00); profiles/hbm_traffic_c3_c5.md.
+# Counters cannot be read from inside the timed run, so the figure is carried here.
+MEASURED_TRAFFIC_BYTES = {"c3": (2.050 + 0.504) * 2**30, "c5": (3.442 + 0.032) * 2**30, "decode": 3.568 * 2**30}
+
 WORKLOADS = {
     # name: B, T(M), N, H, D, gate mean, gate std, head_first, fwd_only, seq_start
     "c2": dict(B=4, M=512, N=512, H=12, D=64, mean=0.0, std=1.0, head_first=False, fwd_only=False, pad=False),
     "c3": dict(B=4, M=16384, N=16384, H=16, D=128, mean=3.0, std=1.0, head_first=False, fwd_only=False, pad=False),
     "c4": dict(B=4, M=16384, N=16384, H=16, D=128, mean=-1.0, std=2.0, head_first=False, fwd_only=False, pad=False),
     "c5": dict(B=16, M=128, N=32768, H=16, D=128, mean=2.0, std=1.0, head_first=True, fwd_only=True, pad=True),
+    # one new token against the same cache (the reference's M == 1 path, ops/forgetting_attention.py:148-153)
+    "decode": dict(B=16, M=1, N=32768, H=16, D=128, mean=2.0, std=1.0, head_first=True, fwd_only=True, pad=True),
 }
 
 
@@ -117,8 +125,11 @@ def stage_times(w, tensors, iters):
     lse = torch.empty((B, H, M), dtype=torch.float32, device=dev)
     o = torch.empty_like(q)
     ss = None if seq_start is None else seq_start.data_ptr()
+    ws_bytes = C.c_int64(0)
+    _lib.check(lib.fox_attn_fwd_workspace_bytes(C.byref(dims), C.byref(ws_bytes)), "workspace")
+    ws = torch.empty(max(ws_bytes.value, 16), dtype=torch.uint8, device=dev)  # key-split partials (prefill / decode shapes)
     fwd = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), c.data_ptr(), lse.data_ptr(), ss, None,
-                       1.0 / math.sqrt(D), None)
+                       1.0 / math.sqrt(D), None, ws.data_ptr() if ws_bytes.value else None, ws_bytes.value)
     out = {}
 
     def scan():
@@ -299,10 +310,21 @@ def main():
             e["tflops"] = kern_flops[name] / t * 1e-12
             e["frac_of_peak"] = e["tflops"] / PEAK_BF16_TFLOPS
         kernels[name] = e
-    dom = "fwd" if w["fwd_only"] else "bwd_dkdv"
-    roofline = {"kernel": dom, "bound": "mfma", "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": kernels[dom]["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
-                "avg_launch_ms": kernels[dom]["ms"]}
+    traffic = MEASURED_TRAFFIC_BYTES.get(ns.workload)
+    if w["fwd_only"]:  # few query rows against a long key sequence: one pass over K and V, HBM-bound
+        dom = "fwd"
+        pad = seq_start.float() if seq_start is not None else torch.zeros(w["B"], device="cuda")
+        alg_bytes = ((2.0 * w["H"] * (w["N"] - pad) * w["D"] * 2).sum().item()
+                     + 2 * w["B"] * w["H"] * w["M"] * w["D"] * 2 + w["B"] * w["H"] * w["N"] * 4)
+        gbps = alg_bytes / stages[dom] * 1e-9
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                    "frac": gbps / PEAK_HBM_GBPS, "traffic": traffic, "algorithmic_bytes": alg_bytes,
+                    "avg_launch_ms": kernels[dom]["ms"]}
+    else:
+        dom = "bwd_dkdv"
+        roofline = {"kernel": dom, "bound": "mfma", "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
+                    "unit": "TFLOP/s", "frac": kernels[dom]["tflops"] / PEAK_BF16_TFLOPS, "traffic": traffic,
+                    "algorithmic_flops": kern_flops[dom], "avg_launch_ms": kernels[dom]["ms"]}
 
     line = {
         "metric": "fwd+bwd TFLOP/s & % bf16 MFMA peak, T=16k D=128; ACP speedup vs no-prune",

@@ -354,8 +354,9 @@ def test_config4_pruned(fa):
         assert rel_err(out, base) <= 1e-3     # pruned mass <= e^-10: far below bf16 rounding
 
 
-def test_config5_chunked_prefill(fa):
-    B, H, M, N, D = 16, 16, 128, 32768, 128
+@pytest.mark.parametrize("M", [128, 1])
+def test_config5_chunked_prefill_and_decode(fa, M):
+    B, H, N, D = 16, 16, 32768, 128
     g_ = torch.Generator(device="cuda").manual_seed(5)
     q = torch.randn(B, H, M, D, generator=g_, device="cuda").bfloat16()
     k = torch.randn(B, H, N, D, generator=g_, device="cuda").bfloat16()
