@@ -172,11 +172,11 @@ typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), other counters untouched
 
-template <int D, int ROWS>
+template <int D, int ROWS, int NW = 4>
 struct DirectTileLoader {
   static constexpr int CH = D / 8;
-  static constexpr int NBLK = ROWS * CH / 64;  // 1 KiB blocks per tile
-  static constexpr int PER = (NBLK + 3) / 4;   // blocks per wave (4 waves)
+  static constexpr int NBLK = ROWS * CH / 64;        // 1 KiB blocks per tile
+  static constexpr int PER = (NBLK + NW - 1) / NW;   // blocks per wave (NW waves)
   static_assert(ROWS * CH % 64 == 0, "tile must be a whole number of 1 KiB blocks");
   int voff[PER];
   int wave;
@@ -184,10 +184,10 @@ struct DirectTileLoader {
   __device__ __forceinline__ DirectTileLoader(int64_t row_stride, int wave_, int lane) : wave(wave_) {
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      // physical slot of this lane inside block (wave + 4j) -> the (row, chunk) stored there
+      // physical slot of this lane inside block (wave + NW*j) -> the (row, chunk) stored there
       const int line = lane >> 4, q = (lane & 15) ^ (line << 2);
       const int p = line * 16 + q;
-      const int row = (wave + 4 * j) * Tile<D>::RPB + p / CH, c = p % CH;
+      const int row = (wave + NW * j) * Tile<D>::RPB + p / CH, c = p % CH;
       voff[j] = (int)(row * row_stride * 2) + (c << 4);
     }
   }
@@ -197,8 +197,8 @@ struct DirectTileLoader {
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, (int)bytes, 0x00020000);
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const int blk = wave + 4 * j;
-      if (NBLK % 4 == 0 || blk < NBLK)
+      const int blk = wave + NW * j;
+      if (NBLK % NW == 0 || blk < NBLK)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(tile + blk * Tile<D>::BLOCK_BYTES), 16, voff[j], 0, 0, 0);
     }
   }
