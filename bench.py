@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Forgetting Attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode|shift] [--no-extras] [--no-cpu-baseline]
 
 A step is one forward + backward pass of ``forgetting_attention`` over one batch
 of synthetic input already resident in HBM (forward only for c5).  The default
@@ -253,12 +253,60 @@ def prefill_report(steps, warmup):
             "frac_of_8TBps": (kv_bytes + other) / t * 1e-9 / PEAK_HBM_GBPS}
 
 
+def shift_report(ns):
+    """Token shift (the key/value pre-processing of the FoX layer) at the training-layer shape:
+    forward + backward, HBM-bound; one JSON line of its own."""
+    from forgetting_transformer import token_shift
+    from forgetting_transformer.ops import _lib
+    from forgetting_transformer.ops.token_shift import _args
+
+    B, T, H, D = 4, 16384, 16, 128
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(B, T, H, D, generator=g, device="cuda").bfloat16().requires_grad_()
+    dout = torch.randn(B, T, H, D, generator=g, device="cuda").bfloat16()
+    curr = torch.rand(B, T, H, generator=g, device="cuda").requires_grad_()
+
+    def step():
+        out = token_shift(x, 1.0 - curr, curr)
+        out.backward(dout)
+        x.grad = curr.grad = None
+    sec = time_steps(step, ns.steps, ns.warmup)
+
+    lib = _lib.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    xd, cd = x.detach(), curr.detach()
+    pd = 1.0 - cd
+    out, dx = torch.empty_like(xd), torch.empty_like(xd)
+    dp, dc = torch.empty_like(cd), torch.empty_like(cd)
+    fwd_args = _args(xd, pd, cd, out=out)
+    bwd_args = _args(xd, pd, cd, dout=dout, dx=dx, dprev_weight=dp, dcurr_weight=dc)
+    t_f = event_time(lambda: _lib.check(lib.fox_token_shift_fwd(C.byref(fwd_args), stream), "shift fwd"), max(5, ns.steps))
+    t_b = event_time(lambda: _lib.check(lib.fox_token_shift_bwd(C.byref(bwd_args), stream), "shift bwd"), max(5, ns.steps))
+    S, W = B * T * H * D * 2, B * T * H * 4
+    bytes_f, bytes_b = 2 * S + 2 * W, 3 * S + 4 * W
+    kernels = {"shift_fwd": {"ms": t_f * 1e3, "gbps": bytes_f / t_f * 1e-9, "algorithmic_bytes": bytes_f},
+               "shift_bwd": {"ms": t_b * 1e3, "gbps": bytes_b / t_b * 1e-9, "algorithmic_bytes": bytes_b}}
+    value = (bytes_f + bytes_b) / sec * 1e-9
+    line = {
+        "metric": "token shift fwd+bwd, algorithmic HBM GB/s (operator incl. autograd and the 1 - curr elementwise op)",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": ns.steps, "warmup": ns.warmup, "ms_per_step": sec * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"shift: B{B} T{T} H{H} D{D} bf16 fwd+bwd, weights fp32 (B,T,H)"},
+        "roofline": {"kernel": "shift_bwd", "bound": "hbm", "achieved": kernels["shift_bwd"]["gbps"], "peak": PEAK_HBM_GBPS,
+                     "unit": "GB/s", "frac": kernels["shift_bwd"]["gbps"] / PEAK_HBM_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get("shift"), "algorithmic_bytes": bytes_b,
+                     "avg_launch_ms": t_b * 1e3},
+        "kernels": kernels,
+    }
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift"])
     ap.add_argument("--no-extras", action="store_true", help="skip the ACP and chunked-prefill reports")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -279,6 +327,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if ns.workload == "shift":
+        return shift_report(ns)
 
     w = WORKLOADS[ns.workload]
     tensors = synth(w, "cuda")

@@ -91,6 +91,37 @@ int make_bwd(const fox_bwd_args* args, fox::BwdK& k, bool need_grads) {
   return FOX_OK;
 }
 
+int make_shift(const fox_shift_args* a, fox::ShiftK& k, bool bwd) {
+  if (!a) return fail(FOX_E_ARG, "args is NULL");
+  if (a->B <= 0 || a->T <= 0 || a->H <= 0) return fail(FOX_E_ARG, "B, T, H must be positive (got %d, %d, %d)", a->B, a->T, a->H);
+  if (a->D != 16 && a->D != 32 && a->D != 64 && a->D != 128) return fail(FOX_E_ARG, "head dim must be one of 16, 32, 64, 128 (got %d)", a->D);
+  if (a->dtype != FOX_DTYPE_BF16 && a->dtype != FOX_DTYPE_FP16) return fail(FOX_E_ARG, "dtype must be FOX_DTYPE_BF16 or FOX_DTYPE_FP16 (got %d)", a->dtype);
+  if (a->B > 65535) return fail(FOX_E_ARG, "B must not exceed 65535");
+  if (!a->x || !a->prev_weight || !a->curr_weight) return fail(FOX_E_ARG, "x, prev_weight and curr_weight must not be NULL");
+  if ((a->x_stride_b & 7) || (a->x_stride_t & 7) || (a->x_stride_h & 7)) return fail(FOX_E_ALIGN, "strides of x must be multiples of 8 elements");
+  const void* vec[4] = {a->x, bwd ? a->dout : a->out, bwd ? a->dx : a->out, a->x};
+  for (const void* p : vec) {
+    if (!p) return fail(FOX_E_ARG, bwd ? "dout and dx must not be NULL" : "out must not be NULL");
+    if (((uintptr_t)p & 15) != 0) return fail(FOX_E_ALIGN, "x, out, dout and dx must be 16-byte aligned");
+  }
+  if (bwd && (!a->dprev_weight || !a->dcurr_weight)) return fail(FOX_E_ARG, "dprev_weight and dcurr_weight must not be NULL");
+  if (!bwd && a->out == a->x) return fail(FOX_E_ARG, "out must not alias x");
+  if (bwd && (a->dx == a->dout || a->dx == a->x)) return fail(FOX_E_ARG, "dx must not alias dout or x");
+  k = fox::ShiftK{};
+  k.x = (const uint16_t*)a->x;
+  k.out = (uint16_t*)a->out;
+  k.dout = (const uint16_t*)a->dout;
+  k.dx = (uint16_t*)a->dx;
+  k.prev_w = a->prev_weight;
+  k.curr_w = a->curr_weight;
+  k.dprev_w = a->dprev_weight;
+  k.dcurr_w = a->dcurr_weight;
+  k.x_sb = a->x_stride_b; k.x_st = a->x_stride_t; k.x_sh = a->x_stride_h;
+  k.w_sb = a->w_stride_b; k.w_st = a->w_stride_t; k.w_sh = a->w_stride_h;
+  k.B = a->B; k.T = a->T; k.H = a->H;
+  return FOX_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -106,6 +137,18 @@ int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_b
   if (kv_block_n) *kv_block_n = fox::kKvBN;
   if (kv_block_m) *kv_block_m = fox::kKvBM;
   return FOX_OK;
+}
+
+int fox_token_shift_fwd(const fox_shift_args* args, void* stream) {
+  fox::ShiftK k;
+  FOX_TRY(make_shift(args, k, false));
+  return check_hip(fox::launch_shift_fwd(k, args->D, args->dtype, (hipStream_t)stream), "fox_token_shift_fwd");
+}
+
+int fox_token_shift_bwd(const fox_shift_args* args, void* stream) {
+  fox::ShiftK k;
+  FOX_TRY(make_shift(args, k, true));
+  return check_hip(fox::launch_shift_bwd(k, args->D, args->dtype, (hipStream_t)stream), "fox_token_shift_bwd");
 }
 
 int fox_cumsum_fwd(const float* g, int64_t g_sb, int64_t g_sh, int64_t g_sn, const int64_t* seq_start, float* c, int32_t B,

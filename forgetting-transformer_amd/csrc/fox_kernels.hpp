@@ -39,6 +39,21 @@ struct BwdK {
   int n_tiles;
 };
 
+// Token shift: x, out, dout, dx are (B, T, H, D) 16-bit with shared element strides; the weights and
+// their gradients are (B, T, H) fp32 with shared element strides.
+struct ShiftK {
+  const uint16_t* x;
+  uint16_t* out;
+  const uint16_t* dout;
+  uint16_t* dx;
+  const float* prev_w;
+  const float* curr_w;
+  float* dprev_w;
+  float* dcurr_w;
+  int64_t x_sb, x_st, x_sh, w_sb, w_st, w_sh;
+  int B, T, H;
+};
+
 // Tile sizes (see fox_tile_config in the public header)
 constexpr int kFwdBM = 128;
 constexpr int kFwdBN = 64;
@@ -50,6 +65,8 @@ int fwd_key_splits(int B, int H, int M, int N);
 hipError_t launch_bwd_delta(const BwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_bwd_dkdv(const BwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_bwd_dq(const BwdK& a, int D, int dtype, hipStream_t s);
+hipError_t launch_shift_fwd(const ShiftK& a, int D, int dtype, hipStream_t s);
+hipError_t launch_shift_bwd(const ShiftK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_cumsum_fwd(const float* g, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start, float* c, int B,
                              int H, int N, hipStream_t s);
 hipError_t launch_cumsum_bwd(const float* dc, float* dg, int B, int H, int N, hipStream_t s);

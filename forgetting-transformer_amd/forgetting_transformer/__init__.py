@@ -6,6 +6,7 @@ Same import path and call signature as the reference package
     from forgetting_transformer import forgetting_attention
 """
 from .ops.forgetting_attention import forgetting_attention
+from .ops.token_shift import token_shift
 
 __version__ = "0.1.0"
-__all__ = ["forgetting_attention"]
+__all__ = ["forgetting_attention", "token_shift"]

@@ -55,6 +55,23 @@ class BwdArgs(C.Structure):
     ]
 
 
+class ShiftArgs(C.Structure):
+    _fields_ = [
+        ("B", C.c_int32), ("T", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
+        ("dtype", C.c_int32),
+        ("x", C.c_void_p),
+        ("x_stride_b", C.c_int64), ("x_stride_t", C.c_int64), ("x_stride_h", C.c_int64),
+        ("prev_weight", C.c_void_p),
+        ("curr_weight", C.c_void_p),
+        ("w_stride_b", C.c_int64), ("w_stride_t", C.c_int64), ("w_stride_h", C.c_int64),
+        ("out", C.c_void_p),
+        ("dout", C.c_void_p),
+        ("dx", C.c_void_p),
+        ("dprev_weight", C.c_void_p),
+        ("dcurr_weight", C.c_void_p),
+    ]
+
+
 # every symbol include/fox_attn.h declares: name -> (restype, argtypes)
 SIGNATURES = {
     "fox_version": (C.c_int, []),
@@ -71,6 +88,8 @@ SIGNATURES = {
     "fox_attn_bwd_dkdv": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),
     "fox_attn_bwd_dq": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),
     "fox_attn_bwd": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),
+    "fox_token_shift_fwd": (C.c_int, [C.POINTER(ShiftArgs), C.c_void_p]),
+    "fox_token_shift_bwd": (C.c_int, [C.POINTER(ShiftArgs), C.c_void_p]),
 }
 
 _lib = None

@@ -136,6 +136,43 @@ int fox_attn_bwd_dkdv(const fox_bwd_args* args, void* stream);
 int fox_attn_bwd_dq(const fox_bwd_args* args, void* stream);
 int fox_attn_bwd(const fox_bwd_args* args, void* stream);
 
+/*
+ * Token shift, the data-dependent mix of every key / value row with its predecessor that the FoX
+ * layer applies in front of the attention (ShiftLinear, model/forgetting_transformer/
+ * modeling_forgetting_transformer.py:68-95).  x, out, dout, dx are 16-bit (B, T, H, D) tensors that
+ * share one set of element strides (unit stride for D, 16-byte aligned, strides multiples of 8);
+ * prev_weight, curr_weight and their gradients are fp32 (B, T, H) tensors that share one set of
+ * element strides.  D is one of 16, 32, 64, 128.  No buffer may alias another.
+ */
+typedef struct fox_shift_args {
+  int32_t B, T, H, D;
+  int32_t dtype;                      /* FOX_DTYPE_* of x, out, dout, dx */
+  const void* x;
+  int64_t x_stride_b, x_stride_t, x_stride_h;
+  const float* prev_weight;
+  const float* curr_weight;
+  int64_t w_stride_b, w_stride_t, w_stride_h;
+  void* out;                          /* written by fox_token_shift_fwd */
+  const void* dout;                   /* backward only */
+  void* dx;                           /* written by fox_token_shift_bwd */
+  float* dprev_weight;                /* written by fox_token_shift_bwd */
+  float* dcurr_weight;                /* written by fox_token_shift_bwd */
+} fox_shift_args;
+
+/*
+ * out[b,t,h,:] = x[b,t,h,:] * curr_weight[b,t,h] + x[b,t-1,h,:] * prev_weight[b,t,h], with x[b,-1] = 0,
+ * evaluated in fp32 and rounded once.  Replaces shift_fwd_kernel as launched by TokenShift.forward
+ * (model/forgetting_transformer/token_shift.py:21-71, :160-191).
+ */
+int fox_token_shift_fwd(const fox_shift_args* args, void* stream);
+
+/*
+ * dx[b,t,h,:] = dout[b,t,h,:] * curr_weight[b,t,h] + dout[b,t+1,h,:] * prev_weight[b,t+1,h],
+ * dcurr_weight[b,t,h] = sum_d dout[b,t,h,d] * x[b,t,h,d], dprev_weight[b,t,h] = sum_d dout[b,t,h,d] * x[b,t-1,h,d].
+ * Replaces shift_bwd_kernel as launched by TokenShift.backward (token_shift.py:83-156, :193-233).
+ */
+int fox_token_shift_bwd(const fox_shift_args* args, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -18,6 +18,11 @@
  *   fox_oracle_find_start_index  :695-745   two-pointer scan, first key block each query block must visit
  *   fox_oracle_find_end_index    :747-795   two-pointer scan, first query row from which a key block is prunable
  *
+ * and (src/forgetting_transformer/model/forgetting_transformer/token_shift.py):
+ *   fox_oracle_token_shift_fwd   :21-71     out[t] = x[t]*curr[t] + x[t-1]*prev[t], x[-1] = 0
+ *   fox_oracle_token_shift_bwd   :83-156    dx[t] = dout[t]*curr[t] + dout[t+1]*prev[t+1]; dcurr = <dout[t], x[t]>;
+ *                                           dprev = <dout[t], x[t-1]>
+ *
  * Layouts: q,out,dout,dq are (B,H,M,D); k,v,dk,dv are (B,H,N,D); c,dc,dg are (B,H,N);
  * lse is (B,H,M); all contiguous.  Build: make -C oracle
  */
@@ -182,4 +187,40 @@ void fox_oracle_find_end_index(const float* c, float threshold, int M, int N, in
     }
     out[o++] = end;
   }
+}
+
+
+/* Token shift: x, out, dout, dx are (B,T,H,D) contiguous doubles; weights and their gradients (B,T,H). */
+void fox_oracle_token_shift_fwd(const double* x, const double* prev_w, const double* curr_w, double* out, int B, int T, int H,
+                                int D) {
+  for (int b = 0; b < B; ++b)
+    for (int t = 0; t < T; ++t)
+      for (int h = 0; h < H; ++h) {
+        const int64_t w = ((int64_t)b * T + t) * H + h;
+        for (int d = 0; d < D; ++d) {
+          const double cur = x[w * D + d];
+          const double before = t > 0 ? x[(w - H) * D + d] : 0.0;
+          out[w * D + d] = cur * curr_w[w] + before * prev_w[w];
+        }
+      }
+}
+
+void fox_oracle_token_shift_bwd(const double* x, const double* prev_w, const double* curr_w, const double* dout, double* dx,
+                                double* dprev_w, double* dcurr_w, int B, int T, int H, int D) {
+  for (int b = 0; b < B; ++b)
+    for (int t = 0; t < T; ++t)
+      for (int h = 0; h < H; ++h) {
+        const int64_t w = ((int64_t)b * T + t) * H + h;
+        double sc = 0.0, sp = 0.0;
+        for (int d = 0; d < D; ++d) {
+          const double g = dout[w * D + d];
+          const double g_after = t + 1 < T ? dout[(w + H) * D + d] : 0.0;
+          const double p_after = t + 1 < T ? prev_w[w + H] : 0.0;
+          dx[w * D + d] = g * curr_w[w] + g_after * p_after;
+          sc += g * x[w * D + d];
+          sp += g * (t > 0 ? x[(w - H) * D + d] : 0.0);
+        }
+        dcurr_w[w] = sc;
+        dprev_w[w] = sp;
+      }
 }

@@ -22,6 +22,12 @@ Reference lines restated here (paths relative to the reference checkout):
 * ``:902-943, 956-1143, 1156-1344, 390-392`` -- the manual backward
   (``manual_backward`` below), written from the kernels' arithmetic.
 
+* ``src/forgetting_transformer/model/forgetting_transformer/token_shift.py:264-270``
+  -- the pure-PyTorch token shift inside its ``test_op`` (``token_shift_ref``):
+  roll by one step, zero the first step, weighted sum in fp32, cast.  Pinned by
+  the identity / pure-shift special cases, an explicit loop, ``gradcheck`` in
+  fp64 and the C restatement.
+
 Pinned by (see tests/test_oracle_cpu.py): ``scaled_dot_product_attention`` with
 an additive mask, ``torch.logsumexp``, the ``g == 0`` and constant-``g``
 closed forms, ``torch.autograd.gradcheck`` in fp64, the identities
@@ -36,6 +42,7 @@ from typing import Optional, Tuple, Union
 import torch
 
 __all__ = [
+    "token_shift_ref",
     "cumulative_log_decay",
     "auto_threshold",
     "forgetting_attention_ref",
@@ -257,3 +264,14 @@ def find_end_index_ref(c_row, threshold: float, M: int, N: int, block_m: int, bl
                 break
         out.append(end)
     return out
+
+
+def token_shift_ref(x: torch.Tensor, prev_weight: torch.Tensor, curr_weight: torch.Tensor) -> torch.Tensor:
+    """``x[b,t-1] * prev_weight[b,t] + x[b,t] * curr_weight[b,t]`` per head with ``x[b,-1] = 0``
+    (reference ``token_shift.py:264-270``).  x: (B, T, H, D); weights: (B, T, H).  The sum is formed
+    in the promoted dtype of x and the weights and cast back to x's dtype; differentiable."""
+    x_prev = torch.roll(x, shifts=1, dims=1)
+    keep = torch.ones(x.shape[1], dtype=torch.bool, device=x.device)
+    keep[0] = False
+    x_prev = torch.where(keep[None, :, None, None], x_prev, torch.zeros_like(x_prev))
+    return (x_prev * prev_weight[..., None] + x * curr_weight[..., None]).to(x.dtype)

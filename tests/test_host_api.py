@@ -59,6 +59,41 @@ def test_c_abi_rejects_bad_arguments_before_launching():
         _lib.check(-1, "x")
 
 
+def test_token_shift_c_abi_and_wrapper_checks():
+    lib = _lib.load()
+    buf = (C.c_char * 4096)()
+    base = C.addressof(buf)
+    base += (-base) % 16
+
+    def args(D=64, dtype=0, x=base, out=base + 1024, xs=(512, 64, 64), dout=None, dx=None, dprev=None, dcurr=None):
+        return _lib.ShiftArgs(1, 2, 1, D, dtype, x, *xs, base + 2048, base + 2304, 2, 1, 1, out, dout, dx, dprev, dcurr)
+
+    assert lib.fox_token_shift_fwd(C.byref(args(D=48)), None) == -1 and b"head dim" in lib.fox_last_error()
+    assert lib.fox_token_shift_fwd(C.byref(args(dtype=3)), None) == -1 and b"dtype" in lib.fox_last_error()
+    assert lib.fox_token_shift_fwd(C.byref(args(x=None)), None) == -1
+    assert lib.fox_token_shift_fwd(C.byref(args(out=None)), None) == -1 and b"out" in lib.fox_last_error()
+    assert lib.fox_token_shift_fwd(C.byref(args(out=base)), None) == -1 and b"alias" in lib.fox_last_error()
+    assert lib.fox_token_shift_fwd(C.byref(args(x=base + 2)), None) == -2
+    assert lib.fox_token_shift_fwd(C.byref(args(xs=(512, 60, 64))), None) == -2 and b"strides" in lib.fox_last_error()
+    assert lib.fox_token_shift_bwd(C.byref(args()), None) == -1            # dout, dx missing
+    assert lib.fox_token_shift_bwd(C.byref(args(dout=base + 1024, dx=base + 1024, dprev=base, dcurr=base)), None) == -1
+    assert lib.fox_token_shift_fwd(None, None) == -1 and lib.fox_token_shift_bwd(None, None) == -1
+
+    from forgetting_transformer import token_shift
+    x = torch.randn(2, 8, 2, 64).bfloat16()
+    w = torch.rand(2, 8, 2)
+    with pytest.raises(AssertionError):
+        token_shift(torch.randn(2, 8, 2, 48).bfloat16(), w, w)            # head dim (token_shift.py:164)
+    with pytest.raises(AssertionError):
+        token_shift(x, w[:, :4], w)                                        # weight shape (:165)
+    with pytest.raises(AssertionError):
+        token_shift(x, w.transpose(0, 1).contiguous().transpose(0, 1), w)  # weight strides differ (:166)
+    with pytest.raises(AssertionError):
+        token_shift(x.float(), w, w)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        token_shift(x, w, w)
+
+
 def test_workspace_query():
     lib = _lib.load()
     need = C.c_int64(-1)

@@ -325,3 +325,52 @@ def test_golden_fixture_is_reproduced():
     bias = (c[..., :, None] - c[..., None, :]).masked_fill(~torch.tril(torch.ones(T, T, dtype=torch.bool)), float("-inf"))
     o2 = ref(q.transpose(1, 2).double(), k.transpose(1, 2).double(), v.transpose(1, 2).double(), attn_mask=bias, scale=1 / 8)
     assert np.allclose(o2.transpose(1, 2).numpy(), data["out"], atol=1e-5)
+
+
+# --------------------------------------------------------------------------------------
+# token shift
+# --------------------------------------------------------------------------------------
+def _shift_inputs(B=2, T=7, H=3, D=4, seed=0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, T, H, D, generator=g, dtype=dtype)
+    curr = torch.rand(B, T, H, generator=g, dtype=dtype)
+    prev = torch.rand(B, T, H, generator=g, dtype=dtype)
+    return x, prev, curr
+
+
+def test_token_shift_special_cases():
+    x, prev, curr = _shift_inputs()
+    one, zero = torch.ones_like(curr), torch.zeros_like(curr)
+    assert torch.equal(O.token_shift_ref(x, zero, one), x)                      # identity
+    shifted = O.token_shift_ref(x, one, zero)                                    # pure shift by one step
+    assert torch.equal(shifted[:, 1:], x[:, :-1]) and shifted[:, 0].abs().max() == 0
+    # explicit loop over every element
+    out = O.token_shift_ref(x, prev, curr)
+    B, T, H, D = x.shape
+    for b in range(B):
+        for t in range(T):
+            for h in range(H):
+                want = x[b, t, h] * curr[b, t, h] + (x[b, t - 1, h] * prev[b, t, h] if t > 0 else 0.0)
+                assert torch.allclose(out[b, t, h], want, rtol=1e-14, atol=0)
+    # linear in x
+    x2, _, _ = _shift_inputs(seed=1)
+    assert torch.allclose(O.token_shift_ref(2.0 * x - x2, prev, curr), 2.0 * out - O.token_shift_ref(x2, prev, curr), atol=1e-12)
+
+
+def test_token_shift_gradcheck_and_c_restatement(c_oracle):
+    x, prev, curr = _shift_inputs(B=2, T=9, H=2, D=8)
+    x, prev, curr = (t.requires_grad_() for t in (x, prev, curr))
+    assert torch.autograd.gradcheck(O.token_shift_ref, (x, prev, curr), eps=1e-6, atol=1e-6)
+    g = torch.Generator().manual_seed(9)
+    dout = torch.randn(x.shape, generator=g, dtype=torch.float64)
+    out = O.token_shift_ref(x, prev, curr)
+    dx, dprev, dcurr = torch.autograd.grad(out, (x, prev, curr), dout)
+    B, T, H, D = x.shape
+    xn, pn, cn, gn = (t.detach().numpy().copy() for t in (x, prev, curr, dout))
+    out_c, dx_c = np.empty_like(xn), np.empty_like(xn)
+    dp_c, dc_c = np.empty_like(pn), np.empty_like(pn)
+    c_oracle.fox_oracle_token_shift_fwd(_dptr(xn), _dptr(pn), _dptr(cn), _dptr(out_c), B, T, H, D)
+    c_oracle.fox_oracle_token_shift_bwd(_dptr(xn), _dptr(pn), _dptr(cn), _dptr(gn), _dptr(dx_c), _dptr(dp_c), _dptr(dc_c),
+                                        B, T, H, D)
+    for got, want in ((out_c, out), (dx_c, dx), (dp_c, dprev), (dc_c, dcurr)):
+        assert np.allclose(got, want.detach().numpy(), rtol=1e-12, atol=1e-12)
