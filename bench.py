@@ -138,6 +138,19 @@ def stage_times(w, tensors, iters):
     def f():
         _lib.check(lib.fox_attn_fwd(C.byref(fwd), stream), "fwd")
 
+    # the same prologue from bf16 gate logits with logsigmoid fused in (forgetting_attention_from_logits)
+    logits = torch.randn(log_fgate.shape, device=dev).bfloat16()
+    if not w["head_first"]:
+        logits = logits.transpose(1, 2).contiguous().transpose(1, 2)
+    lg = torch.empty_like(c)
+
+    def gate_scan():
+        _lib.check(lib.fox_gate_cumsum_fwd(logits.data_ptr(), _lib.DTYPE_BF16, *logits.stride(), ss, lg.data_ptr(), c.data_ptr(),
+                                           B, H, N, stream), "gate scan")
+
+    gate_scan()
+    out["gate_cumsum_fwd"] = event_time(gate_scan, iters)
+    out["torch_logsigmoid"] = event_time(lambda: torch.nn.functional.logsigmoid(logits.float()), iters)
     scan()
     out["cumsum_fwd"] = event_time(scan, iters)
     out["fwd"] = event_time(f, iters)

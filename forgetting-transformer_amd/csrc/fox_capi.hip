@@ -158,6 +158,25 @@ int fox_cumsum_fwd(const float* g, int64_t g_sb, int64_t g_sh, int64_t g_sn, con
   return check_hip(fox::launch_cumsum_fwd(g, g_sb, g_sh, g_sn, seq_start, c, B, H, N, (hipStream_t)stream), "fox_cumsum_fwd");
 }
 
+int fox_gate_cumsum_fwd(const void* logits, int32_t logits_dtype, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start,
+                        float* log_fgate, float* c, int32_t B, int32_t H, int32_t N, void* stream) {
+  if (!logits || !c) return fail(FOX_E_ARG, "logits and c must not be NULL");
+  if (B <= 0 || H <= 0 || N <= 0) return fail(FOX_E_ARG, "B, H, N must be positive");
+  if (logits_dtype < FOX_DTYPE_BF16 || logits_dtype > FOX_DTYPE_FP32) return fail(FOX_E_ARG, "logits_dtype must be FOX_DTYPE_BF16, FP16 or FP32 (got %d)", logits_dtype);
+  return check_hip(fox::launch_gate_cumsum_fwd(logits, logits_dtype, sb, sh, sn, seq_start, log_fgate, c, B, H, N, (hipStream_t)stream),
+                   "fox_gate_cumsum_fwd");
+}
+
+int fox_gate_cumsum_bwd(const float* dc, const void* logits, int32_t logits_dtype, int64_t sb, int64_t sh, int64_t sn,
+                        void* dlogits, int64_t db, int64_t dh, int64_t dn, int32_t B, int32_t H, int32_t N, void* stream) {
+  if (!dc || !logits || !dlogits) return fail(FOX_E_ARG, "dc, logits and dlogits must not be NULL");
+  if (B <= 0 || H <= 0 || N <= 0) return fail(FOX_E_ARG, "B, H, N must be positive");
+  if (logits_dtype < FOX_DTYPE_BF16 || logits_dtype > FOX_DTYPE_FP32) return fail(FOX_E_ARG, "logits_dtype must be FOX_DTYPE_BF16, FP16 or FP32 (got %d)", logits_dtype);
+  if ((const void*)dc == dlogits || logits == dlogits) return fail(FOX_E_ARG, "dlogits must not alias dc or logits");
+  return check_hip(fox::launch_gate_cumsum_bwd(dc, logits, logits_dtype, sb, sh, sn, dlogits, db, dh, dn, B, H, N, (hipStream_t)stream),
+                   "fox_gate_cumsum_bwd");
+}
+
 int fox_cumsum_bwd(const float* dc, float* dg, int32_t B, int32_t H, int32_t N, void* stream) {
   if (!dc || !dg) return fail(FOX_E_ARG, "dc and dg must not be NULL");
   if (B <= 0 || H <= 0 || N <= 0) return fail(FOX_E_ARG, "B, H, N must be positive");

@@ -2,6 +2,7 @@
 //
 //   scan_kernel<false> : c[n]  = sum_{l<=n} g[l], with g[l] := 0 for l < seq_start
 //   scan_kernel<true>  : dg[l] = sum_{n>=l} dc[n]
+//   gate_scan_fwd/bwd  : the same two scans fused with logsigmoid of the gate logits and its derivative
 //   norm_max_kernel / threshold_kernel : the "auto" threshold from the largest row
 //                        L2 norms of q and k.
 //
@@ -13,21 +14,13 @@
 
 namespace fox {
 
-template <bool REVERSE>
-__global__ __launch_bounds__(256) void scan_kernel(const float* __restrict__ in, int64_t sb, int64_t sh, int64_t sn,
-                                                   const int64_t* __restrict__ seq_start, float* __restrict__ out, int H,
-                                                   int N) {
+// Scan of one row: element idx is produced by load(idx) and the running sum up to and including
+// it is handed to store(idx, sum).  REVERSE walks the row from its last element to its first.
+template <bool REVERSE, typename Load, typename Store>
+__device__ __forceinline__ void scan_row(int N, Load load, Store store) {
   constexpr int PER = 4, NT = 256, SPAN = PER * NT;
   __shared__ double wave_tot[NT / kWave];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int bh = blockIdx.x, b = bh / H, h = bh % H;
-  const float* src = in + b * sb + h * sh;
-  float* dst = out + (int64_t)bh * N;
-  int seq = 0;
-  if (!REVERSE && seq_start) {
-    const int64_t s64 = seq_start[b];
-    seq = (int)(s64 < 0 ? 0 : (s64 > N ? N : s64));
-  }
   double carry = 0.0;
   for (int base = 0; base < N; base += SPAN) {
     double v[PER];
@@ -37,7 +30,7 @@ __global__ __launch_bounds__(256) void scan_kernel(const float* __restrict__ in,
       const int pos = base + tid * PER + e;            // position in scan order
       const int idx = REVERSE ? N - 1 - pos : pos;     // element index
       float x = 0.f;
-      if (pos < N && (REVERSE || idx >= seq)) x = src[(int64_t)idx * sn];
+      if (pos < N) x = load(idx);
       run += (double)x;
       v[e] = run;
     }
@@ -62,11 +55,113 @@ __global__ __launch_bounds__(256) void scan_kernel(const float* __restrict__ in,
     for (int e = 0; e < PER; ++e) {
       const int pos = base + tid * PER + e;
       const int idx = REVERSE ? N - 1 - pos : pos;
-      if (pos < N) dst[idx] = (float)(before + v[e]);
+      if (pos < N) store(idx, (float)(before + v[e]));
     }
     carry += total;
     __syncthreads();
   }
+}
+
+template <bool REVERSE>
+__global__ __launch_bounds__(256) void scan_kernel(const float* __restrict__ in, int64_t sb, int64_t sh, int64_t sn,
+                                                   const int64_t* __restrict__ seq_start, float* __restrict__ out, int H,
+                                                   int N) {
+  const int bh = blockIdx.x, b = bh / H, h = bh % H;
+  const float* src = in + b * sb + h * sh;
+  float* dst = out + (int64_t)bh * N;
+  int seq = 0;
+  if (!REVERSE && seq_start) {
+    const int64_t s64 = seq_start[b];
+    seq = (int)(s64 < 0 ? 0 : (s64 > N ? N : s64));
+  }
+  scan_row<REVERSE>(
+      N, [&](int idx) { return (REVERSE || idx >= seq) ? src[(int64_t)idx * sn] : 0.f; },
+      [&](int idx, float sum) { dst[idx] = sum; });
+}
+
+// Forget-gate logits in fp32, bf16 or fp16 (the output of the gate projection of the FoX layer).
+template <int DT>
+__device__ __forceinline__ float load_logit(const void* p, int64_t i) {
+  if constexpr (DT == 2) return reinterpret_cast<const float*>(p)[i];
+  const uint32_t w = reinterpret_cast<const uint16_t*>(p)[i];
+  if constexpr (DT == 0) return Bf16::lo(w);
+  return Fp16::lo(w);
+}
+template <int DT>
+__device__ __forceinline__ void store_logit(void* p, int64_t i, float x) {
+  if constexpr (DT == 2) reinterpret_cast<float*>(p)[i] = x;
+  else if constexpr (DT == 0) reinterpret_cast<uint16_t*>(p)[i] = (uint16_t)(Bf16::pack2(x, 0.f) & 0xffffu);
+  else reinterpret_cast<uint16_t*>(p)[i] = (uint16_t)(Fp16::pack2(x, 0.f) & 0xffffu);
+}
+
+// c[n] = sum_{seq_start <= l <= n} logsigmoid(x[l]) in one pass over the logits; optionally also
+// stores log_fgate[n] = logsigmoid(x[n]) (the decode cache of the FoX layer keeps it).
+template <int DT>
+__global__ __launch_bounds__(256) void gate_scan_fwd_kernel(const void* __restrict__ logits, int64_t sb, int64_t sh, int64_t sn,
+                                                            const int64_t* __restrict__ seq_start,
+                                                            float* __restrict__ log_fgate, float* __restrict__ out, int H,
+                                                            int N) {
+  const int bh = blockIdx.x, b = bh / H, h = bh % H;
+  const int64_t base = b * sb + h * sh;
+  float* dst = out + (int64_t)bh * N;
+  float* lg = log_fgate ? log_fgate + (int64_t)bh * N : nullptr;
+  int seq = 0;
+  if (seq_start) {
+    const int64_t s64 = seq_start[b];
+    seq = (int)(s64 < 0 ? 0 : (s64 > N ? N : s64));
+  }
+  scan_row<false>(
+      N,
+      [&](int idx) {
+        const float x = load_logit<DT>(logits, base + (int64_t)idx * sn);
+        const float g = fminf(x, 0.f) - log1pf(expf(-fabsf(x)));  // logsigmoid, stable on both sides
+        if (lg) lg[idx] = g;
+        return idx >= seq ? g : 0.f;
+      },
+      [&](int idx, float sum) { dst[idx] = sum; });
+}
+
+// dlogit[l] = (sum_{n>=l} dc[n]) * d logsigmoid(x_l)/dx = dg[l] * (1 - sigmoid(x_l)), stored in the
+// dtype and layout of the logits.
+template <int DT>
+__global__ __launch_bounds__(256) void gate_scan_bwd_kernel(const float* __restrict__ dc, const void* __restrict__ logits,
+                                                            int64_t sb, int64_t sh, int64_t sn, void* __restrict__ dlogits,
+                                                            int64_t db, int64_t dh, int64_t dn, int H, int N) {
+  const int bh = blockIdx.x, b = bh / H, h = bh % H;
+  const float* src = dc + (int64_t)bh * N;
+  const int64_t lbase = b * sb + h * sh, dbase = b * db + h * dh;
+  scan_row<true>(
+      N, [&](int idx) { return src[idx]; },
+      [&](int idx, float sum) {
+        const float x = load_logit<DT>(logits, lbase + (int64_t)idx * sn);
+        const float z = expf(-fabsf(x));
+        const float r = z / (1.f + z);                       // sigmoid(-|x|)
+        store_logit<DT>(dlogits, dbase + (int64_t)idx * dn, sum * (x < 0.f ? 1.f - r : r));
+      });
+}
+
+hipError_t launch_gate_cumsum_fwd(const void* logits, int dtype, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start,
+                                  float* log_fgate, float* c, int B, int H, int N, hipStream_t s) {
+  const dim3 grid((unsigned)(B * H));
+  switch (dtype) {
+    case 0: hipLaunchKernelGGL(gate_scan_fwd_kernel<0>, grid, dim3(256), 0, s, logits, sb, sh, sn, seq_start, log_fgate, c, H, N); break;
+    case 1: hipLaunchKernelGGL(gate_scan_fwd_kernel<1>, grid, dim3(256), 0, s, logits, sb, sh, sn, seq_start, log_fgate, c, H, N); break;
+    case 2: hipLaunchKernelGGL(gate_scan_fwd_kernel<2>, grid, dim3(256), 0, s, logits, sb, sh, sn, seq_start, log_fgate, c, H, N); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_gate_cumsum_bwd(const float* dc, const void* logits, int dtype, int64_t sb, int64_t sh, int64_t sn,
+                                  void* dlogits, int64_t db, int64_t dh, int64_t dn, int B, int H, int N, hipStream_t s) {
+  const dim3 grid((unsigned)(B * H));
+  switch (dtype) {
+    case 0: hipLaunchKernelGGL(gate_scan_bwd_kernel<0>, grid, dim3(256), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
+    case 1: hipLaunchKernelGGL(gate_scan_bwd_kernel<1>, grid, dim3(256), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
+    case 2: hipLaunchKernelGGL(gate_scan_bwd_kernel<2>, grid, dim3(256), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
 }
 
 hipError_t launch_cumsum_fwd(const float* g, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start, float* c, int B,

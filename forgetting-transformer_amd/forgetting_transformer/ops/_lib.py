@@ -13,6 +13,7 @@ LIB_PATH = Path(__file__).resolve().parent.parent / "_lib" / "libfox_attn.so"
 
 DTYPE_BF16 = 0
 DTYPE_FP16 = 1
+DTYPE_FP32 = 2  # gate logits only
 
 
 class View(C.Structure):
@@ -80,6 +81,10 @@ SIGNATURES = {
     "fox_cumsum_fwd": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                  C.c_int32, C.c_void_p]),
     "fox_cumsum_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
+    "fox_gate_cumsum_fwd": (C.c_int, [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                      C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
+    "fox_gate_cumsum_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int64,
+                                      C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "fox_auto_threshold": (C.c_int, [C.POINTER(Dims), C.POINTER(View), C.POINTER(View), C.c_float, C.c_void_p, C.c_void_p,
                                      C.c_void_p]),
     "fox_attn_fwd": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),

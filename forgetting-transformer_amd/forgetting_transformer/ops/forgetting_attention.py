@@ -20,7 +20,8 @@ import torch
 
 from . import _lib
 
-__all__ = ["forgetting_attention", "ForgettingAttention"]
+__all__ = ["forgetting_attention", "forgetting_attention_from_logits", "ForgettingAttention",
+           "ForgettingAttentionFromLogits"]
 
 _DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
 
@@ -61,135 +62,189 @@ class ForgettingAttention(torch.autograd.Function):
     def forward(ctx, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
                 return_log_normalizer=False, return_start_index=False, record_time_key=None,
                 record_attention_time=False, record_find_index_time=False):
-        assert causal, "Only causal attention is supported"
-        assert not (record_attention_time or record_find_index_time), \
-            "in-op timers are not implemented; profile the kernels with rocprofv3 instead"
-        Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
-        assert Dq == Dk == Dv, "feature size of q, k, v should be equal"
-        assert Dk in {16, 32, 64, 128}, "We only support head dims in {16, 32, 64, 128}"
-        assert q.dtype == k.dtype == v.dtype, "q, k, v must share one dtype"
-
-        B, H, M, D = q.shape
-        N = k.shape[2]
-        assert log_fgate.shape == (B, H, N)
-        assert log_fgate.dtype == torch.float32, (
-            "log_fgate must be in torch.float32. It is best to do this cast before logsigmoid, "
-            "e.g., torch.nn.functional.logsigmoid(fgate_logit.float()).")
-        if sm_scale is None:
-            sm_scale = 1.0 / math.sqrt(D)
-        sm_scale = float(sm_scale)
-
-        Hk, Hv = k.shape[1], v.shape[1]
-        assert Hk == Hv, "num of heads in k and v should be equal"
-        assert H == Hk, "groupped query attention has not been tested. You can uncomment this if you know what you are doing."
-        assert k.shape == (B, Hk, N, D) and v.shape == (B, Hv, N, D)
-        assert not (M > N), "The key/value tensors must be longer than the query tensor"
-
-        # threshold: validate on the host first (:91-109), compute "auto" on the device later
-        auto_threshold = False
-        if adaptive_threshold is not None:
-            if isinstance(adaptive_threshold, str):
-                assert adaptive_threshold == "auto", (
-                    'adaptive_threshold must be either the string "auto", a float, or a Tensor, '
-                    f"but got {adaptive_threshold}.")
-                auto_threshold = True
-            else:
-                adaptive_threshold = torch.as_tensor(adaptive_threshold, dtype=torch.float, device=q.device)
-                try:
-                    adaptive_threshold = torch.broadcast_to(adaptive_threshold, (B, H))
-                except RuntimeError:
-                    raise RuntimeError(
-                        'adaptive_threshold must be either the string "auto" or broadcastable to '
-                        f"(batch_size, num_heads) = ({B}, {H}), but got {adaptive_threshold.size()}.")
-                assert adaptive_threshold.size() == (B, H)
-                adaptive_threshold = adaptive_threshold.contiguous()
-
-        if seq_start is not None:
-            has_seq_start = True
-            assert seq_start.shape == (B,)
-        else:
-            has_seq_start = False
-
-        if q.device.type != "cuda":
-            raise RuntimeError("forgetting_attention runs only on an AMD GPU (HIP device); "
-                               f"got tensors on '{q.device}'. There is no CPU implementation.")
-        lib = _lib.load()
-        device = q.device
-        dims = _lib.Dims(B, H, M, N, D, _DTYPES[q.dtype])
-        if has_seq_start:
-            seq_start = seq_start.to(device=device, dtype=torch.long).contiguous()
-
-        q, k, v = maybe_contiguous(q), maybe_contiguous(k), maybe_contiguous(v)
-
-        with torch.cuda.device(device):
-            stream = _stream(device)
-
-            if auto_threshold:
-                adaptive_threshold = torch.empty((B, H), dtype=torch.float32, device=device)
-                scratch = torch.empty((B, H, 2), dtype=torch.int32, device=device)
-                qv, kv = _view(q), _view(k)
-                _lib.check(lib.fox_auto_threshold(C.byref(dims), C.byref(qv), C.byref(kv), sm_scale,
-                                                  _ptr(adaptive_threshold), _ptr(scratch), stream), "fox_auto_threshold")
-
-            # c = cumsum(log_fgate) with gates left of seq_start zeroed, one fused kernel
-            log_lambda = torch.empty((B, H, N), dtype=torch.float32, device=device)
-            _lib.check(lib.fox_cumsum_fwd(_ptr(log_fgate), log_fgate.stride(0), log_fgate.stride(1), log_fgate.stride(2),
-                                          _ptr(seq_start), _ptr(log_lambda), B, H, N, stream), "fox_cumsum_fwd")
-
-            o = torch.empty_like(q)
-            L = torch.empty((B, H, M), device=device, dtype=torch.float32)
-            first_block = None
-            if return_start_index:
-                block_m, _, _, _ = _lib.tile_config(D)
-                first_block = torch.zeros((B, H, (M + block_m - 1) // block_m), dtype=torch.int32, device=device)
-            ws_bytes = C.c_int64(0)
-            _lib.check(lib.fox_attn_fwd_workspace_bytes(C.byref(dims), C.byref(ws_bytes)), "fox_attn_fwd_workspace_bytes")
-            workspace = torch.empty(ws_bytes.value, dtype=torch.uint8, device=device) if ws_bytes.value > 0 else None
-            args = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), log_lambda.data_ptr(), L.data_ptr(),
-                                None if seq_start is None else seq_start.data_ptr(),
-                                None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
-                                sm_scale, None if first_block is None else first_block.data_ptr(),
-                                None if workspace is None else workspace.data_ptr(), ws_bytes.value)
-            _lib.check(lib.fox_attn_fwd(C.byref(args), stream), "fox_attn_fwd")
-
-        ctx.save_for_backward(q, k, v, o, L, log_lambda, seq_start, adaptive_threshold)
-        ctx.sm_scale = sm_scale
-        ctx.causal = causal
-        ctx.has_seq_start = has_seq_start
-
-        if return_log_normalizer or return_start_index:
-            start_index = None
-            if return_start_index:
-                _, block_n, _, _ = _lib.tile_config(D)
-                start_index = first_block.to(torch.long) * block_n
-            outs = (o, L if return_log_normalizer else None, start_index)
-            ctx.mark_non_differentiable(*[t for t in outs[1:] if t is not None])
-            return outs
-        return o
+        return _forward(ctx, False, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
+                        return_log_normalizer, return_start_index, record_attention_time, record_find_index_time)
 
     @staticmethod
     def backward(ctx, do, *ignored):
-        q, k, v, o, L, log_lambda, seq_start, adaptive_threshold = ctx.saved_tensors
-        B, H, M, D = q.shape
-        N = k.shape[2]
-        device = q.device
-        lib = _lib.load()
-        do = maybe_contiguous(do)
-        with torch.cuda.device(device):
-            stream = _stream(device)
-            delta = torch.empty_like(L)
-            dlog_lambda = torch.empty((B, H, N), dtype=torch.float32, device=device)
-            dlog_fgate = torch.empty((B, H, N), dtype=torch.float32, device=device)
-            dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-            args = _lib.BwdArgs(
-                _lib.Dims(B, H, M, N, D, _DTYPES[q.dtype]),
-                _view(q), _view(k), _view(v), _view(o), _view(do), _view(dq), _view(dk), _view(dv),
-                log_lambda.data_ptr(), L.data_ptr(),
-                None if seq_start is None else seq_start.data_ptr(),
-                None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
-                ctx.sm_scale, delta.data_ptr(), dlog_lambda.data_ptr(), dlog_fgate.data_ptr())
+        return _backward(ctx, do) + (None,) * 9
+
+
+class ForgettingAttentionFromLogits(torch.autograd.Function):
+    """The same operator fed with the forget-gate *logits*: ``logsigmoid`` (fp32) is fused into the
+    cumulative-sum kernel and its derivative into the reverse scan of the backward, which removes the
+    layer's separate ``logsigmoid(fgate_logit.float())`` pass
+    (``modeling_forgetting_transformer.py:343-346``).  Returns ``(out, log_fgate)``; ``log_fgate``
+    (fp32, what the decode cache stores) is not differentiable here."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, fgate_logit, seq_start, sm_scale, adaptive_threshold):
+        out = _forward(ctx, True, q, k, v, fgate_logit, seq_start, True, sm_scale, adaptive_threshold,
+                       False, False, False, False)
+        ctx.mark_non_differentiable(ctx.log_fgate)
+        return out, ctx.log_fgate
+
+    @staticmethod
+    def backward(ctx, do, *ignored):
+        return _backward(ctx, do) + (None,) * 3
+
+
+_GATE_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16, torch.float32: _lib.DTYPE_FP32}
+
+
+def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
+             return_log_normalizer, return_start_index, record_attention_time, record_find_index_time):
+    assert causal, "Only causal attention is supported"
+    assert not (record_attention_time or record_find_index_time), \
+        "in-op timers are not implemented; profile the kernels with rocprofv3 instead"
+    Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
+    assert Dq == Dk == Dv, "feature size of q, k, v should be equal"
+    assert Dk in {16, 32, 64, 128}, "We only support head dims in {16, 32, 64, 128}"
+    assert q.dtype == k.dtype == v.dtype, "q, k, v must share one dtype"
+
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    assert log_fgate.shape == (B, H, N)
+    if gate_is_logit:
+        assert log_fgate.dtype in _GATE_DTYPES, "the gate logits must be bfloat16, float16 or float32"
+    else:
+        assert log_fgate.dtype == torch.float32, (
+            "log_fgate must be in torch.float32. It is best to do this cast before logsigmoid, "
+            "e.g., torch.nn.functional.logsigmoid(fgate_logit.float()).")
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    sm_scale = float(sm_scale)
+
+    Hk, Hv = k.shape[1], v.shape[1]
+    assert Hk == Hv, "num of heads in k and v should be equal"
+    assert H == Hk, "groupped query attention has not been tested. You can uncomment this if you know what you are doing."
+    assert k.shape == (B, Hk, N, D) and v.shape == (B, Hv, N, D)
+    assert not (M > N), "The key/value tensors must be longer than the query tensor"
+
+    # threshold: validate on the host first (:91-109), compute "auto" on the device later
+    auto_threshold = False
+    if adaptive_threshold is not None:
+        if isinstance(adaptive_threshold, str):
+            assert adaptive_threshold == "auto", (
+                'adaptive_threshold must be either the string "auto", a float, or a Tensor, '
+                f"but got {adaptive_threshold}.")
+            auto_threshold = True
+        else:
+            adaptive_threshold = torch.as_tensor(adaptive_threshold, dtype=torch.float, device=q.device)
+            try:
+                adaptive_threshold = torch.broadcast_to(adaptive_threshold, (B, H))
+            except RuntimeError:
+                raise RuntimeError(
+                    'adaptive_threshold must be either the string "auto" or broadcastable to '
+                    f"(batch_size, num_heads) = ({B}, {H}), but got {adaptive_threshold.size()}.")
+            assert adaptive_threshold.size() == (B, H)
+            adaptive_threshold = adaptive_threshold.contiguous()
+
+    if seq_start is not None:
+        has_seq_start = True
+        assert seq_start.shape == (B,)
+    else:
+        has_seq_start = False
+
+    if q.device.type != "cuda":
+        raise RuntimeError("forgetting_attention runs only on an AMD GPU (HIP device); "
+                           f"got tensors on '{q.device}'. There is no CPU implementation.")
+    lib = _lib.load()
+    device = q.device
+    dims = _lib.Dims(B, H, M, N, D, _DTYPES[q.dtype])
+    if has_seq_start:
+        seq_start = seq_start.to(device=device, dtype=torch.long).contiguous()
+
+    q, k, v = maybe_contiguous(q), maybe_contiguous(k), maybe_contiguous(v)
+
+    with torch.cuda.device(device):
+        stream = _stream(device)
+
+        if auto_threshold:
+            adaptive_threshold = torch.empty((B, H), dtype=torch.float32, device=device)
+            scratch = torch.empty((B, H, 2), dtype=torch.int32, device=device)
+            qv, kv = _view(q), _view(k)
+            _lib.check(lib.fox_auto_threshold(C.byref(dims), C.byref(qv), C.byref(kv), sm_scale,
+                                              _ptr(adaptive_threshold), _ptr(scratch), stream), "fox_auto_threshold")
+
+        # c = cumsum(log_fgate) with gates left of seq_start zeroed, one fused kernel
+        log_lambda = torch.empty((B, H, N), dtype=torch.float32, device=device)
+        if gate_is_logit:  # logsigmoid fused into the scan; the fp32 log gates are a by-product
+            ctx.log_fgate = torch.empty((B, H, N), dtype=torch.float32, device=device)
+            _lib.check(lib.fox_gate_cumsum_fwd(_ptr(log_fgate), _GATE_DTYPES[log_fgate.dtype], log_fgate.stride(0),
+                                               log_fgate.stride(1), log_fgate.stride(2), _ptr(seq_start),
+                                               _ptr(ctx.log_fgate), _ptr(log_lambda), B, H, N, stream),
+                       "fox_gate_cumsum_fwd")
+        else:
+            _lib.check(lib.fox_cumsum_fwd(_ptr(log_fgate), log_fgate.stride(0), log_fgate.stride(1),
+                                          log_fgate.stride(2), _ptr(seq_start), _ptr(log_lambda), B, H, N, stream),
+                       "fox_cumsum_fwd")
+
+        o = torch.empty_like(q)
+        L = torch.empty((B, H, M), device=device, dtype=torch.float32)
+        first_block = None
+        if return_start_index:
+            block_m, _, _, _ = _lib.tile_config(D)
+            first_block = torch.zeros((B, H, (M + block_m - 1) // block_m), dtype=torch.int32, device=device)
+        ws_bytes = C.c_int64(0)
+        _lib.check(lib.fox_attn_fwd_workspace_bytes(C.byref(dims), C.byref(ws_bytes)), "fox_attn_fwd_workspace_bytes")
+        workspace = torch.empty(ws_bytes.value, dtype=torch.uint8, device=device) if ws_bytes.value > 0 else None
+        args = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), log_lambda.data_ptr(), L.data_ptr(),
+                            None if seq_start is None else seq_start.data_ptr(),
+                            None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
+                            sm_scale, None if first_block is None else first_block.data_ptr(),
+                            None if workspace is None else workspace.data_ptr(), ws_bytes.value)
+        _lib.check(lib.fox_attn_fwd(C.byref(args), stream), "fox_attn_fwd")
+
+    ctx.save_for_backward(q, k, v, o, L, log_lambda, seq_start, adaptive_threshold,
+                          log_fgate if gate_is_logit else None)
+    ctx.sm_scale = sm_scale
+    ctx.causal = causal
+    ctx.has_seq_start = has_seq_start
+
+    if return_log_normalizer or return_start_index:
+        start_index = None
+        if return_start_index:
+            _, block_n, _, _ = _lib.tile_config(D)
+            start_index = first_block.to(torch.long) * block_n
+        outs = (o, L if return_log_normalizer else None, start_index)
+        ctx.mark_non_differentiable(*[t for t in outs[1:] if t is not None])
+        return outs
+    return o
+
+def _backward(ctx, do):
+    q, k, v, o, L, log_lambda, seq_start, adaptive_threshold, gate_logit = ctx.saved_tensors
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    device = q.device
+    lib = _lib.load()
+    do = maybe_contiguous(do)
+    with torch.cuda.device(device):
+        stream = _stream(device)
+        delta = torch.empty_like(L)
+        dlog_lambda = torch.empty((B, H, N), dtype=torch.float32, device=device)
+        dlog_fgate = torch.empty((B, H, N), dtype=torch.float32, device=device) if gate_logit is None else None
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        args = _lib.BwdArgs(
+            _lib.Dims(B, H, M, N, D, _DTYPES[q.dtype]),
+            _view(q), _view(k), _view(v), _view(o), _view(do), _view(dq), _view(dk), _view(dv),
+            log_lambda.data_ptr(), L.data_ptr(),
+            None if seq_start is None else seq_start.data_ptr(),
+            None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
+            ctx.sm_scale, delta.data_ptr(), dlog_lambda.data_ptr(), None if dlog_fgate is None else dlog_fgate.data_ptr())
+        if gate_logit is None:
             _lib.check(lib.fox_attn_bwd(C.byref(args), stream), "fox_attn_bwd")
-        return dq, dk, dv, dlog_fgate, None, None, None, None, None, None, None, None, None
+            dgate = dlog_fgate
+        else:  # same stages, the last one fused with the derivative of logsigmoid
+            _lib.check(lib.fox_attn_bwd_delta(C.byref(args), stream), "fox_attn_bwd_delta")
+            _lib.check(lib.fox_attn_bwd_dkdv(C.byref(args), stream), "fox_attn_bwd_dkdv")
+            _lib.check(lib.fox_attn_bwd_dq(C.byref(args), stream), "fox_attn_bwd_dq")
+            dgate = torch.empty_like(gate_logit)
+            _lib.check(lib.fox_gate_cumsum_bwd(_ptr(dlog_lambda), _ptr(gate_logit), _GATE_DTYPES[gate_logit.dtype],
+                                               gate_logit.stride(0), gate_logit.stride(1), gate_logit.stride(2),
+                                               _ptr(dgate), dgate.stride(0), dgate.stride(1), dgate.stride(2), B, H, N,
+                                               stream), "fox_gate_cumsum_bwd")
+    return dq, dk, dv, dgate
 
 
 def forgetting_attention(
@@ -238,3 +293,36 @@ def forgetting_attention(
     if not head_first:
         out = out.transpose(1, 2)
     return out
+
+
+def forgetting_attention_from_logits(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    fgate_logit: torch.Tensor,
+    *,
+    head_first: bool = False,
+    seq_start: Optional[torch.Tensor] = None,
+    sm_scale: Optional[float] = None,
+    adaptive_threshold: Optional[Union[Literal["auto"], float, torch.Tensor]] = None,
+):
+    """``forgetting_attention(q, k, v, logsigmoid(fgate_logit.float()), ...)`` with the log-sigmoid fused into
+    the operator's scan kernels (forward and backward).
+
+    ``fgate_logit`` is the output of the layer's gate projection, (batch, seqlen_k, heads) unless
+    head_first=True, in bfloat16, float16 or float32; every other argument is as in
+    ``forgetting_attention``.  Returns ``(out, log_fgate)`` where ``log_fgate`` is the float32
+    ``logsigmoid(fgate_logit)`` in the layout of ``fgate_logit`` (what the layer's decode cache
+    stores, ``modeling_forgetting_transformer.py:356-357``); gradients flow to q, k, v and
+    fgate_logit through ``out`` only.
+    """
+    for name, entry in dict(q=q, k=k, v=v).items():
+        assert entry.dtype in [torch.float16, torch.bfloat16], (
+            f"Only torch.float16 or torch.bfloat16 are supported for q/k/v, but got {entry.dtype} for {name}.")
+    if not head_first:
+        q, k, v = [item.transpose(1, 2) for item in (q, k, v)]
+        fgate_logit = fgate_logit.transpose(1, 2)
+    out, log_fgate = ForgettingAttentionFromLogits.apply(q, k, v, fgate_logit, seq_start, sm_scale, adaptive_threshold)
+    if not head_first:
+        out, log_fgate = out.transpose(1, 2), log_fgate.transpose(1, 2)
+    return out, log_fgate

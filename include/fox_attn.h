@@ -31,6 +31,7 @@ extern "C" {
 
 #define FOX_DTYPE_BF16 0
 #define FOX_DTYPE_FP16 1
+#define FOX_DTYPE_FP32 2   /* gate logits only */
 
 /* A (B, H, T, D) tensor view: element strides of the first three axes. */
 typedef struct fox_view {
@@ -69,6 +70,24 @@ int fox_cumsum_fwd(const float* g, int64_t g_sb, int64_t g_sh, int64_t g_sn, con
  * Replaces the reverse cumulative sum at :390-392.
  */
 int fox_cumsum_bwd(const float* dc, float* dg, int32_t B, int32_t H, int32_t N, void* stream);
+
+/*
+ * The prologue of the FoX layer fused with the scan: c[b,h,n] = sum_{seq_start[b] <= l <= n} logsigmoid(x[b,h,l])
+ * from the gate logits x (dtype FOX_DTYPE_BF16 / FP16 / FP32, element strides (sb, sh, sn)), evaluated in fp32.
+ * Replaces logsigmoid(fgate_logit.float()) of the layer (model/forgetting_transformer/
+ * modeling_forgetting_transformer.py:343-346) followed by the operator's prologue (:117-127).  log_fgate, if
+ * not NULL, receives logsigmoid(x) as (B,H,N) contiguous fp32 (the layer's decode cache stores it,
+ * modeling_forgetting_transformer.py:356-357).
+ */
+int fox_gate_cumsum_fwd(const void* logits, int32_t logits_dtype, int64_t sb, int64_t sh, int64_t sn,
+                        const int64_t* seq_start, float* log_fgate, float* c, int32_t B, int32_t H, int32_t N, void* stream);
+
+/*
+ * dlogits[b,h,l] = (sum_{n>=l} dc[b,h,n]) * (1 - sigmoid(x[b,h,l])): the reverse cumulative sum (:390-392)
+ * fused with the derivative of logsigmoid; dlogits has the dtype of the logits and its own element strides.
+ */
+int fox_gate_cumsum_bwd(const float* dc, const void* logits, int32_t logits_dtype, int64_t sb, int64_t sh, int64_t sn,
+                        void* dlogits, int64_t db, int64_t dh, int64_t dn, int32_t B, int32_t H, int32_t N, void* stream);
 
 /*
  * thr[b,h] = -(2 * max_m|q| * max_n|k| * sm_scale + log N) - 10, with the row norms
