@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Forgetting Attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode|shift] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode|shift|norm_gate] [--no-extras] [--no-cpu-baseline]
 
 A step is one forward + backward pass of ``forgetting_attention`` over one batch
 of synthetic input already resident in HBM (forward only for c5).  The default
@@ -314,12 +314,65 @@ def shift_report(ns):
     print(json.dumps(line))
 
 
+def norm_gate_report(ns):
+    """Gated per-head RMS norm (the FoX layer's epilogue on the attention output) at the training-layer
+    shape: forward + backward, HBM-bound; one JSON line of its own."""
+    from forgetting_transformer import group_norm_gated
+    from forgetting_transformer.ops import _lib
+
+    B, T, G, D = 4, 16384, 16, 128
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(B, T, G * D, generator=gen, device="cuda").bfloat16().requires_grad_()
+    g = torch.randn(B, T, G * D, generator=gen, device="cuda").bfloat16().requires_grad_()
+    dy = torch.randn(B, T, G * D, generator=gen, device="cuda").bfloat16()
+    w = (torch.rand(G * D, generator=gen, device="cuda") + 0.5).requires_grad_()
+
+    def step():
+        y = group_norm_gated(x, g, w, None, "sigmoid", is_rms_norm=True, num_groups=G)
+        y.backward(dy)
+        x.grad = g.grad = w.grad = None
+    sec = time_steps(step, ns.steps, ns.warmup)
+
+    lib = _lib.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rows, width = B * T, G * D
+    xd, gd, wd = x.detach().view(rows, width), g.detach().view(rows, width), w.detach()
+    y, dx, dg = torch.empty_like(xd), torch.empty_like(xd), torch.empty_like(xd)
+    rstd = torch.empty(rows, G, device="cuda")
+    dw = torch.empty(width, device="cuda")
+    nb = C.c_int64(0)
+    _lib.check(lib.fox_norm_gate_workspace_bytes(rows, G, D, C.byref(nb)), "workspace")
+    ws = torch.empty(nb.value, dtype=torch.uint8, device="cuda")
+    args = _lib.NormGateArgs(rows, G, D, _lib.DTYPE_BF16, _lib.ACT_SIGMOID, 1e-6, xd.data_ptr(), width, gd.data_ptr(), width,
+                             wd.data_ptr(), y.data_ptr(), width, rstd.data_ptr(), dy.data_ptr(), width, dx.data_ptr(), width,
+                             dg.data_ptr(), width, dw.data_ptr(), ws.data_ptr())
+    t_f = event_time(lambda: _lib.check(lib.fox_norm_gate_fwd(C.byref(args), stream), "norm fwd"), max(5, ns.steps))
+    t_b = event_time(lambda: _lib.check(lib.fox_norm_gate_bwd(C.byref(args), stream), "norm bwd"), max(5, ns.steps))
+    S = rows * width * 2
+    bytes_f, bytes_b = 3 * S + rows * G * 4, 5 * S + rows * G * 4 + 2 * nb.value
+    kernels = {"norm_gate_fwd": {"ms": t_f * 1e3, "gbps": bytes_f / t_f * 1e-9, "algorithmic_bytes": bytes_f},
+               "norm_gate_bwd": {"ms": t_b * 1e3, "gbps": bytes_b / t_b * 1e-9, "algorithmic_bytes": bytes_b}}
+    line = {
+        "metric": "gated per-head RMS norm fwd+bwd, algorithmic HBM GB/s (operator incl. autograd)",
+        "value": (bytes_f + bytes_b) / sec * 1e-9, "unit": "GB/s", "n_gpus": 1, "steps": ns.steps, "warmup": ns.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"norm_gate: B{B} T{T} heads{G} D{D} bf16 fwd+bwd, sigmoid gate, fp32 weight"},
+        "roofline": {"kernel": "norm_gate_bwd", "bound": "hbm", "achieved": kernels["norm_gate_bwd"]["gbps"],
+                     "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": kernels["norm_gate_bwd"]["gbps"] / PEAK_HBM_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get("norm_gate"), "algorithmic_bytes": bytes_b,
+                     "avg_launch_ms": t_b * 1e3},
+        "kernels": kernels,
+    }
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift", "norm_gate"])
     ap.add_argument("--no-extras", action="store_true", help="skip the ACP and chunked-prefill reports")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -343,6 +396,8 @@ def main():
 
     if ns.workload == "shift":
         return shift_report(ns)
+    if ns.workload == "norm_gate":
+        return norm_gate_report(ns)
 
     w = WORKLOADS[ns.workload]
     tensors = synth(w, "cuda")

@@ -19,7 +19,7 @@ ROOT = Path(__file__).resolve().parent
 CSRC = ROOT / "csrc"
 OBJ_DIR = ROOT / "build"
 LIB_PATH = ROOT / "forgetting_transformer" / "_lib" / "libfox_attn.so"
-SOURCES = ["fox_fwd.hip", "fox_bwd.hip", "fox_scan.hip", "fox_shift.hip", "fox_capi.hip"]
+SOURCES = ["fox_fwd.hip", "fox_bwd.hip", "fox_scan.hip", "fox_shift.hip", "fox_norm_gate.hip", "fox_capi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

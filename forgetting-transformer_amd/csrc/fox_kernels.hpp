@@ -54,6 +54,25 @@ struct ShiftK {
   int B, T, H;
 };
 
+// Gated per-head RMS norm: x, g, y, dy, dx, dg are (R rows, G heads, D) 16-bit, heads and head dim
+// contiguous, each with its own row stride; w, dw are (G*D) fp32; rstd is (R, G) fp32.
+struct NormGateK {
+  const uint16_t* x;
+  const uint16_t* g;
+  uint16_t* y;
+  const uint16_t* dy;
+  uint16_t* dx;
+  uint16_t* dg;
+  const float* w;
+  float* rstd;
+  float* dw;
+  float* dw_partial;
+  int64_t x_sr, g_sr, y_sr, dy_sr, dx_sr, dg_sr;
+  int64_t R;
+  int G;
+  float eps;
+};
+
 // Tile sizes (see fox_tile_config in the public header)
 constexpr int kFwdBM = 128;
 constexpr int kFwdBN = 64;
@@ -65,6 +84,9 @@ int fwd_key_splits(int B, int H, int M, int N);
 hipError_t launch_bwd_delta(const BwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_bwd_dkdv(const BwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_bwd_dq(const BwdK& a, int D, int dtype, hipStream_t s);
+hipError_t launch_norm_gate(const NormGateK& a, int D, int dtype, bool bwd, bool swish, hipStream_t s);
+int64_t norm_gate_strips(int64_t rows);
+int64_t norm_gate_workspace_rows(int64_t rows);
 hipError_t launch_shift_fwd(const ShiftK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_shift_bwd(const ShiftK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_cumsum_fwd(const float* g, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start, float* c, int B,

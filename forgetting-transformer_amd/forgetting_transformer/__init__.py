@@ -6,7 +6,8 @@ Same import path and call signature as the reference package
     from forgetting_transformer import forgetting_attention
 """
 from .ops.forgetting_attention import forgetting_attention, forgetting_attention_from_logits
+from .ops.norm_gate import group_norm_gated
 from .ops.token_shift import token_shift
 
 __version__ = "0.1.0"
-__all__ = ["forgetting_attention", "forgetting_attention_from_logits", "token_shift"]
+__all__ = ["forgetting_attention", "forgetting_attention_from_logits", "group_norm_gated", "token_shift"]

@@ -73,6 +73,30 @@ class ShiftArgs(C.Structure):
     ]
 
 
+ACT_SIGMOID = 0
+ACT_SWISH = 1
+
+
+class NormGateArgs(C.Structure):
+    _fields_ = [
+        ("rows", C.c_int64),
+        ("G", C.c_int32), ("D", C.c_int32),
+        ("dtype", C.c_int32),
+        ("activation", C.c_int32),
+        ("eps", C.c_float),
+        ("x", C.c_void_p), ("x_stride_row", C.c_int64),
+        ("g", C.c_void_p), ("g_stride_row", C.c_int64),
+        ("weight", C.c_void_p),
+        ("y", C.c_void_p), ("y_stride_row", C.c_int64),
+        ("rstd", C.c_void_p),
+        ("dy", C.c_void_p), ("dy_stride_row", C.c_int64),
+        ("dx", C.c_void_p), ("dx_stride_row", C.c_int64),
+        ("dg", C.c_void_p), ("dg_stride_row", C.c_int64),
+        ("dweight", C.c_void_p),
+        ("workspace", C.c_void_p),
+    ]
+
+
 # every symbol include/fox_attn.h declares: name -> (restype, argtypes)
 SIGNATURES = {
     "fox_version": (C.c_int, []),
@@ -93,6 +117,9 @@ SIGNATURES = {
     "fox_attn_bwd_dkdv": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),
     "fox_attn_bwd_dq": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),
     "fox_attn_bwd": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),
+    "fox_norm_gate_fwd": (C.c_int, [C.POINTER(NormGateArgs), C.c_void_p]),
+    "fox_norm_gate_bwd": (C.c_int, [C.POINTER(NormGateArgs), C.c_void_p]),
+    "fox_norm_gate_workspace_bytes": (C.c_int, [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_int64)]),
     "fox_token_shift_fwd": (C.c_int, [C.POINTER(ShiftArgs), C.c_void_p]),
     "fox_token_shift_bwd": (C.c_int, [C.POINTER(ShiftArgs), C.c_void_p]),
 }

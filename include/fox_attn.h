@@ -192,6 +192,50 @@ int fox_token_shift_fwd(const fox_shift_args* args, void* stream);
  */
 int fox_token_shift_bwd(const fox_shift_args* args, void* stream);
 
+/*
+ * Gated per-head RMS normalisation, the epilogue the FoX layer applies to the attention output before the
+ * output projection (FusedGroupNormGated(num_groups=heads, is_rms_norm=True, activation="sigmoid"),
+ * model/forgetting_transformer/modeling_forgetting_transformer.py:243, :417-420):
+ *   y[r,h,:] = x[r,h,:] * rstd[r,h] * weight[h,:] * act(g[r,h,:]),  rstd = 1/sqrt(mean_d x[r,h,:]^2 + eps),
+ * act = sigmoid (FOX_ACT_SIGMOID) or g*sigmoid(g) (FOX_ACT_SWISH).  x, g, y, dy, dx, dg are 16-bit tensors of
+ * `rows` rows of G*D contiguous elements, each with its own row stride in elements (a multiple of 8, base
+ * pointers 16-byte aligned); weight and dweight are G*D fp32; rstd is (rows, G) fp32, written by the
+ * forward and read by the backward.  No bias, no residual.  D is one of 16, 32, 64, 128.
+ */
+#define FOX_ACT_SIGMOID 0
+#define FOX_ACT_SWISH 1
+
+typedef struct fox_norm_gate_args {
+  int64_t rows;
+  int32_t G, D;
+  int32_t dtype;        /* FOX_DTYPE_BF16 / FP16 of the 16-bit tensors */
+  int32_t activation;   /* FOX_ACT_* */
+  float eps;
+  const void* x;  int64_t x_stride_row;
+  const void* g;  int64_t g_stride_row;
+  const float* weight;
+  void* y;        int64_t y_stride_row;    /* written by fox_norm_gate_fwd */
+  float* rstd;
+  const void* dy; int64_t dy_stride_row;   /* backward only from here on */
+  void* dx;       int64_t dx_stride_row;
+  void* dg;       int64_t dg_stride_row;
+  float* dweight;
+  float* workspace;     /* fox_norm_gate_workspace_bytes() bytes, 16-byte aligned */
+} fox_norm_gate_args;
+
+/* Replaces layer_norm_gated_fwd_kernel as launched by LayerNormGatedFunction.forward (fuse_norm_gate.py:132-206, :539-618). */
+int fox_norm_gate_fwd(const fox_norm_gate_args* args, void* stream);
+
+/*
+ * dx, dg and dweight = sum over rows of dy*act(g)*xhat.  Replaces layer_norm_gated_bwd_kernel and the sum over
+ * its partial weight gradients (fuse_norm_gate.py:309-417, :620-724).  The partial sums live in `workspace`
+ * and are added in a fixed order, so the result is reproducible bit for bit.
+ */
+int fox_norm_gate_bwd(const fox_norm_gate_args* args, void* stream);
+
+/* Size of the backward's workspace for `rows` rows of G heads of D elements. */
+int fox_norm_gate_workspace_bytes(int64_t rows, int32_t G, int32_t D, int64_t* bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,10 @@
  *   fox_oracle_token_shift_bwd   :83-156    dx[t] = dout[t]*curr[t] + dout[t+1]*prev[t+1]; dcurr = <dout[t], x[t]>;
  *                                           dprev = <dout[t], x[t-1]>
  *
+ * and (src/forgetting_transformer/model/forgetting_transformer/fuse_norm_gate.py):
+ *   fox_oracle_norm_gate_fwd/bwd :132-206, :309-417  per-group RMS norm * weight * sigmoid(g) (swish = 1: g*sigmoid(g)),
+ *                                           dx, dg, dweight as in the backward kernel
+ *
  * Layouts: q,out,dout,dq are (B,H,M,D); k,v,dk,dv are (B,H,N,D); c,dc,dg are (B,H,N);
  * lse is (B,H,M); all contiguous.  Build: make -C oracle
  */
@@ -223,4 +227,49 @@ void fox_oracle_token_shift_bwd(const double* x, const double* prev_w, const dou
         dcurr_w[w] = sc;
         dprev_w[w] = sp;
       }
+}
+
+
+/* Gated per-group RMS norm: x, g, y, dy, dx, dg are (R, G, D) contiguous doubles; w, dw are (G, D). */
+void fox_oracle_norm_gate_fwd(const double* x, const double* g, const double* w, double* y, int64_t R, int G, int D, double eps,
+                              int swish) {
+  for (int64_t r = 0; r < R; ++r)
+    for (int h = 0; h < G; ++h) {
+      const int64_t o = (r * G + h) * D;
+      double ss = 0.0;
+      for (int d = 0; d < D; ++d) ss += x[o + d] * x[o + d];
+      const double rstd = 1.0 / sqrt(ss / D + eps);
+      for (int d = 0; d < D; ++d) {
+        const double s = 1.0 / (1.0 + exp(-g[o + d]));
+        y[o + d] = x[o + d] * rstd * w[h * D + d] * (swish ? g[o + d] * s : s);
+      }
+    }
+}
+
+void fox_oracle_norm_gate_bwd(const double* x, const double* g, const double* w, const double* dy, double* dx, double* dg,
+                              double* dw, int64_t R, int G, int D, double eps, int swish) {
+  for (int j = 0; j < G * D; ++j) dw[j] = 0.0;
+  for (int64_t r = 0; r < R; ++r)
+    for (int h = 0; h < G; ++h) {
+      const int64_t o = (r * G + h) * D;
+      double ss = 0.0;
+      for (int d = 0; d < D; ++d) ss += x[o + d] * x[o + d];
+      const double rstd = 1.0 / sqrt(ss / D + eps);
+      double c1 = 0.0;
+      for (int d = 0; d < D; ++d) {
+        const double xhat = x[o + d] * rstd, s = 1.0 / (1.0 + exp(-g[o + d]));
+        const double act = swish ? g[o + d] * s : s;
+        const double dact = swish ? s + g[o + d] * s * (1.0 - s) : s * (1.0 - s);
+        dg[o + d] = dy[o + d] * xhat * w[h * D + d] * dact;
+        const double dyn = dy[o + d] * act;
+        dw[h * D + d] += dyn * xhat;
+        c1 += xhat * dyn * w[h * D + d];
+      }
+      c1 /= D;
+      for (int d = 0; d < D; ++d) {
+        const double xhat = x[o + d] * rstd, s = 1.0 / (1.0 + exp(-g[o + d]));
+        const double act = swish ? g[o + d] * s : s;
+        dx[o + d] = (dy[o + d] * act * w[h * D + d] - xhat * c1) * rstd;
+      }
+    }
 }

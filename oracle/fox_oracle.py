@@ -28,6 +28,13 @@ Reference lines restated here (paths relative to the reference checkout):
   the identity / pure-shift special cases, an explicit loop, ``gradcheck`` in
   fp64 and the C restatement.
 
+* ``src/forgetting_transformer/model/forgetting_transformer/fuse_norm_gate.py:18-53``
+  -- ``group_norm_gated_ref`` for the RMS / no bias / no residual case
+  (``group_norm_gated_ref`` here): per-group ``x / sqrt(mean(x^2) + eps) * weight``
+  times ``sigmoid(g)`` (or ``g * sigmoid(g)``), evaluated in the upcast dtype.
+  Pinned by ``torch.nn.functional.rms_norm`` per group, ``gradcheck`` in fp64 and
+  the C restatement.
+
 Pinned by (see tests/test_oracle_cpu.py): ``scaled_dot_product_attention`` with
 an additive mask, ``torch.logsumexp``, the ``g == 0`` and constant-``g``
 closed forms, ``torch.autograd.gradcheck`` in fp64, the identities
@@ -42,6 +49,7 @@ from typing import Optional, Tuple, Union
 import torch
 
 __all__ = [
+    "group_norm_gated_ref",
     "token_shift_ref",
     "cumulative_log_decay",
     "auto_threshold",
@@ -275,3 +283,20 @@ def token_shift_ref(x: torch.Tensor, prev_weight: torch.Tensor, curr_weight: tor
     keep[0] = False
     x_prev = torch.where(keep[None, :, None, None], x_prev, torch.zeros_like(x_prev))
     return (x_prev * prev_weight[..., None] + x * curr_weight[..., None]).to(x.dtype)
+
+
+def group_norm_gated_ref(x: torch.Tensor, g: torch.Tensor, weight: torch.Tensor, num_groups: int, eps: float = 1e-6,
+                         activation: str = "sigmoid", upcast: bool = True) -> torch.Tensor:
+    """Per-group RMS norm with weight, times the gate activation (reference
+    ``fuse_norm_gate.py:18-53`` with ``is_rms_norm=True``, no bias, no residual).  x, g: (..., G*D)."""
+    dtype = x.dtype
+    if upcast and dtype in (torch.float16, torch.bfloat16):
+        x, g, weight = x.float(), g.float(), weight.float()
+    shape = x.shape
+    xg = x.reshape(*shape[:-1], num_groups, shape[-1] // num_groups)
+    wg = weight.reshape(num_groups, shape[-1] // num_groups)
+    rstd = 1 / torch.sqrt(xg.square().mean(dim=-1, keepdim=True) + eps)
+    out = (xg * rstd * wg).reshape(shape)
+    s = torch.sigmoid(g)
+    out = out * (s if activation == "sigmoid" else g * s)
+    return out.to(dtype)

@@ -98,6 +98,48 @@ def test_token_shift_c_abi_and_wrapper_checks():
         token_shift(x, w, w)
 
 
+def test_norm_gate_c_abi_and_wrapper_checks():
+    lib = _lib.load()
+    buf = (C.c_char * 8192)()
+    base = C.addressof(buf)
+    base += (-base) % 16
+
+    def args(D=64, dtype=0, act=0, x=base, y=base + 1024, xs=64, rstd=base + 4096, weight=base + 2048):
+        return _lib.NormGateArgs(2, 1, D, dtype, act, 1e-6, x, xs, base + 512, 64, weight, y, 64, rstd,
+                                 None, 0, None, 0, None, 0, None, None)
+
+    assert lib.fox_norm_gate_fwd(C.byref(args(D=48)), None) == -1 and b"head dim" in lib.fox_last_error()
+    assert lib.fox_norm_gate_fwd(C.byref(args(dtype=2)), None) == -1 and b"dtype" in lib.fox_last_error()
+    assert lib.fox_norm_gate_fwd(C.byref(args(act=5)), None) == -1 and b"activation" in lib.fox_last_error()
+    assert lib.fox_norm_gate_fwd(C.byref(args(x=None)), None) == -1
+    assert lib.fox_norm_gate_fwd(C.byref(args(y=None)), None) == -1 and b"y must not be NULL" in lib.fox_last_error()
+    assert lib.fox_norm_gate_fwd(C.byref(args(x=base + 4)), None) == -2
+    assert lib.fox_norm_gate_fwd(C.byref(args(xs=60)), None) == -2 and b"row strides" in lib.fox_last_error()
+    assert lib.fox_norm_gate_bwd(C.byref(args()), None) == -1        # dy, dx, dg missing
+    assert lib.fox_norm_gate_fwd(None, None) == -1 and lib.fox_norm_gate_bwd(None, None) == -1
+    nb = C.c_int64(0)
+    assert lib.fox_norm_gate_workspace_bytes(65536, 16, 128, C.byref(nb)) == 0
+    assert nb.value == (2048 + 64) * 16 * 128 * 4                     # one row per 32-row strip + one per 32 strips
+    assert lib.fox_norm_gate_workspace_bytes(1, 1, 48, C.byref(nb)) == -1
+    assert lib.fox_norm_gate_workspace_bytes(1, 1, 64, None) == -1
+
+    from forgetting_transformer import group_norm_gated
+    x = torch.randn(4, 128).bfloat16()
+    w = torch.ones(128)
+    with pytest.raises(NotImplementedError):
+        group_norm_gated(x, x, w, torch.zeros(128), "sigmoid", is_rms_norm=True, num_groups=2)
+    with pytest.raises(NotImplementedError):
+        group_norm_gated(x, x, w, None, "sigmoid", residual=x, is_rms_norm=True, num_groups=2)
+    with pytest.raises(ValueError):
+        group_norm_gated(x, x, w, None, "tanh", is_rms_norm=True, num_groups=2)
+    with pytest.raises(AssertionError):
+        group_norm_gated(x, x, w, None, "sigmoid", is_rms_norm=True, num_groups=3)
+    with pytest.raises(AssertionError):
+        group_norm_gated(x.float(), x.float(), w, None, "sigmoid", is_rms_norm=True, num_groups=2)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        group_norm_gated(x, x, w, None, "sigmoid", is_rms_norm=True, num_groups=2)
+
+
 def test_workspace_query():
     lib = _lib.load()
     need = C.c_int64(-1)
