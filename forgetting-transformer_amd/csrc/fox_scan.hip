@@ -18,20 +18,27 @@ namespace fox {
 // it is handed to store(idx, sum).  REVERSE walks the row from its last element to its first.
 template <bool REVERSE, typename Load, typename Store>
 __device__ __forceinline__ void scan_row(int N, Load load, Store store) {
-  constexpr int PER = 4, NT = 256, SPAN = PER * NT;
+  constexpr int PER = 8, NT = 256, SPAN = PER * NT;
   __shared__ double wave_tot[NT / kWave];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   double carry = 0.0;
-  for (int base = 0; base < N; base += SPAN) {
-    double v[PER];
-    double run = 0.0;
+  float x[PER], x_next[PER];
+  auto fetch = [&](int base, float (&dst)[PER]) {  // the elements this thread owns in the span starting at base
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
       const int pos = base + tid * PER + e;            // position in scan order
       const int idx = REVERSE ? N - 1 - pos : pos;     // element index
-      float x = 0.f;
-      if (pos < N) x = load(idx);
-      run += (double)x;
+      dst[e] = pos < N ? load(idx) : 0.f;
+    }
+  };
+  fetch(0, x);
+  for (int base = 0; base < N; base += SPAN) {
+    if (base + SPAN < N) fetch(base + SPAN, x_next);   // in flight while this span is scanned
+    double v[PER];
+    double run = 0.0;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      run += (double)x[e];
       v[e] = run;
     }
     // inclusive scan of the per-thread totals across the wave, then across waves
@@ -58,6 +65,8 @@ __device__ __forceinline__ void scan_row(int N, Load load, Store store) {
       if (pos < N) store(idx, (float)(before + v[e]));
     }
     carry += total;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) x[e] = x_next[e];
     __syncthreads();
   }
 }
@@ -94,6 +103,16 @@ __device__ __forceinline__ void store_logit(void* p, int64_t i, float x) {
   else reinterpret_cast<uint16_t*>(p)[i] = (uint16_t)(Fp16::pack2(x, 0.f) & 0xffffu);
 }
 
+// logsigmoid(x) = min(x, 0) - log1p(exp(-|x|)), stable on both sides, from the hardware exp / log:
+// log1p(z) for z in (0, 1] is log(u) + (z - (u - 1)) / u with u = fl(1 + z), which repairs the rounding
+// of 1 + z (absolute error ~1e-8, and log1p(z) -> z for tiny z as it must).
+__device__ __forceinline__ float log_sigmoid(float x) {
+  const float z = __expf(-fabsf(x));
+  const float u = 1.0f + z;
+  const float l = __logf(u) + __fdividef(z - (u - 1.0f), u);
+  return fminf(x, 0.f) - l;
+}
+
 // c[n] = sum_{seq_start <= l <= n} logsigmoid(x[l]) in one pass over the logits; optionally also
 // stores log_fgate[n] = logsigmoid(x[n]) (the decode cache of the FoX layer keeps it).
 template <int DT>
@@ -114,7 +133,7 @@ __global__ __launch_bounds__(256) void gate_scan_fwd_kernel(const void* __restri
       N,
       [&](int idx) {
         const float x = load_logit<DT>(logits, base + (int64_t)idx * sn);
-        const float g = fminf(x, 0.f) - log1pf(expf(-fabsf(x)));  // logsigmoid, stable on both sides
+        const float g = log_sigmoid(x);
         if (lg) lg[idx] = g;
         return idx >= seq ? g : 0.f;
       },
@@ -134,8 +153,8 @@ __global__ __launch_bounds__(256) void gate_scan_bwd_kernel(const float* __restr
       N, [&](int idx) { return src[idx]; },
       [&](int idx, float sum) {
         const float x = load_logit<DT>(logits, lbase + (int64_t)idx * sn);
-        const float z = expf(-fabsf(x));
-        const float r = z / (1.f + z);                       // sigmoid(-|x|)
+        const float z = __expf(-fabsf(x));
+        const float r = __fdividef(z, 1.f + z);              // sigmoid(-|x|)
         store_logit<DT>(dlogits, dbase + (int64_t)idx * dn, sum * (x < 0.f ? 1.f - r : r));
       });
 }

@@ -18,7 +18,7 @@ def pytest_configure(config):
 
 def make_inputs(B, H, M, N, D, *, dtype=torch.bfloat16, device="cpu", seed=0, gate_mean=0.0, gate_std=1.0,
                 gate_uniform=None, qkv_std=1.0, head_first=True, seq_start=None, requires_grad=False):
-    """Seeded synthetic inputs in the distributions BASELINE's configs name.
+    """Seeded synthetic inputs in the distributions the benchmark configurations name.
 
     Everything is drawn on the CPU in fp32 (so CPU and GPU runs see the same values)
     and then cast / moved.  Returns q, k, v, log_fgate, dout (+ seq_start tensor).

@@ -3,7 +3,7 @@
 The reference holds no fixtures for Forgetting Attention (its only test builds its
 inputs on a CUDA device at run time), so these vectors come from this repository's
 own oracle, whose functions are pinned in tests/test_oracle_cpu.py.  Inputs follow
-BASELINE's first config: B=2, T=256, H=4, D=64, q/k/v ~ N(0,1), log_fgate =
+Benchmark configuration 1: B=2, T=256, H=4, D=64, q/k/v ~ N(0,1), log_fgate =
 logsigmoid(N(0,1)), sm_scale = 1/8, (batch, time, head, dim) layout, fp32.
 A second file holds a small bf16 forward+backward case with left padding and
 seqlen_q < seqlen_k, including gradients, for the GPU parity test.

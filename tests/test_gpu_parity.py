@@ -2,7 +2,7 @@
 operator, against the oracle on the same seeded inputs.
 
 Tolerance (bf16): max |x - ref| <= 2e-2 * max(1, max|ref|) for out, dq, dk, dv,
-dlog_fgate, the bound BASELINE states ("max-abs error 2e-2 relative to output scale",
+dlog_fgate, the bound the benchmark configurations are judged by ("max-abs error 2e-2 relative to output scale",
 with the scale floored at 1 so that a reference that is zero up to rounding -- a row with
 a single valid key has dS = 0 exactly -- does not turn rounding noise into a relative error).  The
 reference's own grid (fp16) uses its own bound, atol = 1e-2
@@ -80,7 +80,7 @@ def test_golden_forward_backward(fa):
 
 
 def test_golden_c1_shape(fa):
-    """BASELINE config 1 (B2 T256 H4 D64, sm_scale 1/8): same inputs rounded to bf16."""
+    """Benchmark configuration 1 (B2 T256 H4 D64, sm_scale 1/8): same inputs rounded to bf16."""
     d = np.load(ROOT / "tests" / "golden" / "c1_b2_t256_h4_d64.npz")
     q, k, v = (torch.from_numpy(d[n]).cuda().bfloat16() for n in ("q", "k", "v"))
     g = torch.from_numpy(d["log_fgate"]).cuda()
@@ -96,7 +96,7 @@ def test_golden_c1_shape(fa):
 # --------------------------------------------------------------------------------------
 @pytest.mark.parametrize("D", [16, 32, 64, 128])
 def test_config2_library_example(fa, D):
-    """BASELINE config 2: B4 T512 H12, bf16 fwd+bwd, (batch, time, head, dim) layout."""
+    """Benchmark configuration 2: B4 T512 H12, bf16 fwd+bwd, (batch, time, head, dim) layout."""
     run_case(fa, 4, 12, 512, 512, D, head_first=False, seed=D)
 
 
@@ -320,7 +320,7 @@ def test_linearity_in_values_and_upstream_gradient(fa):
 
 
 # --------------------------------------------------------------------------------------
-# BASELINE configs 3-5 at full size
+# benchmark configurations 3-5 at full size
 # --------------------------------------------------------------------------------------
 def _full_size_check(fa, B, H, T, D, mean, std, thr, pairs):
     g_ = torch.Generator(device="cuda").manual_seed(3)
