@@ -430,7 +430,9 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     kld.issue(kp, a.k.st, n0, N, kt);
     vld.issue(vp, a.v.st, n0, N, vt);
   };
+  const bool wave_has_rows = m0 + 32 * wave < M;  // a wave without query rows only moves tiles
   auto compute = [&](int n0, const char* kt, const char* vt, const float* cn) {
+    if (!wave_has_rows) return;
     dq_tile<Tr, D>(kt, vt, cn, qreg, doreg, dqacc, rsum, n0, a_m, a_w0, qk_scale, rowc, delta, lane);
   };
 

@@ -280,8 +280,11 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     kld.issue(kp, a.k.st, n0, N, kt);
     vld.issue(vp, a.v.st, n0, N, vt);
   };
+  // A wave whose 32 rows all lie beyond M (decode and other short query blocks) still moves its share
+  // of every tile but computes nothing.
+  const bool wave_has_rows = m0 + 32 * wave < M;
   auto compute = [&](int n0, const char* kt, const char* vt, const float* cn) {
-    if (n0 > a_w0 + 31) return;  // tile entirely above this wave's rows
+    if (n0 > a_w0 + 31 || !wave_has_rows) return;  // tile entirely above this wave's rows
     fwd_tile<Tr, D>(kt, vt, cn, qreg, oacc, m_i, l_i, n0, a_m, qk_scale, lane, n0 + BN - 1 > a_w0);
   };
 
@@ -336,6 +339,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     f32x16 s_a[NB], s_b[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
+      if (!wave_has_rows) break;
       s_a[nb] = acc_init(cn_s0, 32 * nb, g);
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) s_a[nb] = Tr::mfma32(lds_row_operand<D>(k_tile0, 32 * nb + i, 2 * kk + g), qreg[kk], s_a[nb]);
@@ -348,7 +352,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
       __syncthreads();
       if (j + 2 < n_int) issue_k(j + 2, k_tile0);
       if (j + 1 < n_int) issue_v(j + 1, v_tile1);
-      fwd_tile_pipelined<Tr, D>(k_tile1, v_tile0, cn_s1, qreg, oacc, m_i, l_i, qk_scale, lane, s_a, s_b);
+      if (wave_has_rows) fwd_tile_pipelined<Tr, D>(k_tile1, v_tile0, cn_s1, qreg, oacc, m_i, l_i, qk_scale, lane, s_a, s_b);
       if (j + 1 >= n_int) break;
       // odd iteration: K(j+2) in k_tile0 with its key terms in cn_s0, V(j+1) in v_tile1
       wait_vmem_all();
@@ -356,7 +360,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
       __syncthreads();
       if (j + 3 < n_int) issue_k(j + 3, k_tile1);
       if (j + 2 < n_int) issue_v(j + 2, v_tile0);
-      fwd_tile_pipelined<Tr, D>(k_tile0, v_tile1, cn_s0, qreg, oacc, m_i, l_i, qk_scale, lane, s_b, s_a);
+      if (wave_has_rows) fwd_tile_pipelined<Tr, D>(k_tile0, v_tile1, cn_s0, qreg, oacc, m_i, l_i, qk_scale, lane, s_b, s_a);
     }
   }
 
