@@ -10,7 +10,9 @@ from __future__ import annotations
 
 import argparse
 import concurrent.futures
+import json
 import os
+import re
 import subprocess
 import sys
 from pathlib import Path
@@ -19,6 +21,7 @@ ROOT = Path(__file__).resolve().parent
 CSRC = ROOT / "csrc"
 OBJ_DIR = ROOT / "build"
 LIB_PATH = ROOT / "forgetting_transformer" / "_lib" / "libfox_attn.so"
+USAGE_PATH = LIB_PATH.with_name("kernel_resources.json")   # registers, spills, LDS of every kernel, from the compiler
 SOURCES = ["fox_fwd.hip", "fox_bwd.hip", "fox_scan.hip", "fox_shift.hip", "fox_norm_gate.hip", "fox_capi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -26,20 +29,40 @@ FLAGS = [
     # packed fp32 VALU ops are not to be generated for this target
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Rpass-analysis=kernel-resource-usage",   # parsed into kernel_resources.json: the MFMA kernels must not spill
 ]
 
 
-def _compile(src: str) -> Path:
+_REMARK = re.compile(r"remark: (?:\s*)([A-Za-z ]+?)(?: \[bytes/(?:lane|block)\]| \[waves/SIMD\])?: (\S+) \[-Rpass-analysis")
+
+
+def _parse_usage(stderr: str) -> dict:
+    """{mangled kernel name: {"VGPRs": .., "AGPRs": .., "ScratchSize": .., "VGPRs Spill": .., "Occupancy": .., "LDS Size": ..}}"""
+    usage, cur = {}, None
+    for line in stderr.splitlines():
+        m = _REMARK.search(line)
+        if not m:
+            continue
+        key, val = m.group(1).strip(), m.group(2)
+        if key == "Function Name":
+            cur = usage.setdefault(val, {})
+        elif cur is not None and val.lstrip("-").isdigit():
+            cur[key] = int(val)
+    return usage
+
+
+def _compile(src: str):
     obj = OBJ_DIR / (Path(src).stem + ".o")
     cmd = [HIPCC, *FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    noise = ("is not a recognized feature for this target", "-Rpass-analysis=kernel-resource-usage")
+    excerpt = re.compile(r"^\s*\d*\s*\|")   # the source excerpt clang prints under every remark
+    err = "\n".join(l for l in proc.stderr.splitlines() if not any(n in l for n in noise) and not excerpt.match(l))
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{err}")
     if err.strip():
         print(err, file=sys.stderr)
-    return obj
+    return obj, _parse_usage(proc.stderr)
 
 
 def build(jobs: int = 4, force: bool = True) -> Path:
@@ -51,13 +74,16 @@ def build(jobs: int = 4, force: bool = True) -> Path:
         if LIB_PATH.stat().st_mtime >= newest:
             return LIB_PATH
     with concurrent.futures.ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
-        objs = list(ex.map(_compile, SOURCES))
+        results = list(ex.map(_compile, SOURCES))
+    objs = [obj for obj, _ in results]
+    usage = {name: u for _, per_file in results for name, u in per_file.items()}
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--no-undefined", *map(str, objs), "-o", str(LIB_PATH)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stderr}")
     import ctypes
     ctypes.CDLL(str(LIB_PATH), mode=ctypes.RTLD_GLOBAL | getattr(os, "RTLD_NOW", 2))  # every symbol must resolve
+    USAGE_PATH.write_text(json.dumps(usage, indent=1, sort_keys=True))
     return LIB_PATH
 
 

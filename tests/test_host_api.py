@@ -24,6 +24,28 @@ def test_library_exports_every_declared_symbol():
     assert lib.fox_version() >= 100
 
 
+def test_kernels_do_not_spill():
+    """The compiler's resource report, written next to the library by the build: the MFMA kernels must
+    keep every register in the register file (a spill multiplies their run time) at the occupancy
+    they are designed for, and must fit the 160 KiB of LDS of a CU at that occupancy."""
+    import json
+    path = _lib.LIB_PATH.with_name("kernel_resources.json")
+    assert path.exists(), f"{path} is missing: rebuild with python forgetting-transformer_amd/build.py --force"
+    usage = json.loads(path.read_text())
+    want = {"fwd_kernel": 2, "dq_kernel": 2, "dkdv_kernel": 1}          # waves per SIMD
+    seen = set()
+    for name, u in usage.items():
+        for kernel, occupancy in want.items():
+            if f"fox{len(kernel)}{kernel}I" in name.replace("_ZN3", ""):
+                seen.add(kernel)
+                assert u["ScratchSize"] == 0 and u["VGPRs Spill"] == 0, (name, u)
+                assert u["Occupancy"] >= occupancy, (name, u)
+                assert u["LDS Size"] * occupancy <= 160 * 1024, (name, u)
+    assert seen == set(want)
+    for name, u in usage.items():                                        # nothing else spills either
+        assert u["ScratchSize"] == 0, (name, u)
+
+
 def test_tile_config():
     for d in (16, 32, 64, 128):
         bm, bn, kbn, kbm = _lib.tile_config(d)
