@@ -101,84 +101,92 @@ __device__ __forceinline__ void dkdv_step(const char* q_tile, const char* do_til
 //   * the vector arithmetic  P, dS   of block b,
 //   * the accumulation MFMAs dV, dK  of block b-1,
 // which are mutually independent.  A scheduling fence after every chunk keeps the
-// compiler from regrouping them; LDS operands of the next chunk are requested
-// before the fence so their latency hides behind the current chunk.
+// compiler from regrouping them; the LDS operands of a chunk are requested two
+// chunks (about eight MFMAs) ahead, across slot boundaries, so their latency hides
+// behind the chunks in between.
 template <typename Tr, int D>
 __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
                                           const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16],
                                           f32x16 (&dkacc)[(D + 31) / 32], f32x16 (&dvacc)[(D + 31) / 32], float& csum,
                                           float qk_scale, float colc, int lane) {
   constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32, NCH = 8;
+  constexpr int NC = (MB + 2) * NCH;  // chunks of the step: slots -1 .. MB
+  constexpr int PF = 2;               // LDS operands are requested this many chunks before their MFMAs
   static_assert(KK <= NCH && 2 * DB <= NCH, "one k-step and one accumulation pair per chunk");
   const int g = lane >> 5, i = lane & 31;
   f32x16 s[MB], dp[MB];
   u32x4 pb[MB][2], dsb[MB][2];
-#pragma unroll
-  for (int slot = -1; slot <= MB; ++slot) {
-    const bool do_s = slot + 1 < MB, do_v = slot >= 0 && slot < MB, do_c = slot >= 1;
-    const int bs = slot + 1, bv = slot, bc = slot - 1;
-    if (do_s) {  // the accumulators start from the row terms instead of zero
-      s[bs] = acc_init(rc_s, 32 * bs, g);
-      dp[bs] = acc_init(dl_s, 32 * bs, g);
+  u32x4 aq[NC + PF], ado[NC + PF], cq[NC + PF], cdo[NC + PF];  // indexed by chunk; only a few are live at a time
+  auto fetch = [&](auto ic) {
+    constexpr int c = decltype(ic)::value;
+    constexpr int slot = c / NCH - 1, u = c % NCH, bs = slot + 1, bc = slot - 1;
+    if constexpr (c < NC && bs < MB && u < KK) {
+      aq[c] = lds_row_operand<D>(q_tile, 32 * bs + i, 2 * u + g);
+      ado[c] = lds_row_operand<D>(do_tile, 32 * bs + i, 2 * u + g);
     }
-    u32x4 aq[NCH + 1], ado[NCH + 1], cq[NCH + 1], cdo[NCH + 1];
-    auto fetch = [&](int u) {
-      if (do_s && u < KK) {
-        aq[u] = lds_row_operand<D>(q_tile, 32 * bs + i, 2 * u + g);
-        ado[u] = lds_row_operand<D>(do_tile, 32 * bs + i, 2 * u + g);
-      }
-      if (do_c && u < 2 * DB) {
-        cdo[u] = lds_col_operand<D>(do_tile, 32 * bc + 16 * (u / DB), u % DB, lane);
-        cq[u] = lds_col_operand<D>(q_tile, 32 * bc + 16 * (u / DB), u % DB, lane);
-      }
-    };
-    fetch(0);
-#pragma unroll
-    for (int u = 0; u < NCH; ++u) {
-      fetch(u + 1);
-      if (do_s && u < KK) {
-        s[bs] = Tr::mfma32(aq[u], kreg[u], s[bs]);
-        dp[bs] = Tr::mfma32(ado[u], vreg[u], dp[bs]);
-      }
-      if (do_c && u < 2 * DB) {
-        dvacc[u % DB] = Tr::mfma32(cdo[u], pb[bc][u / DB], dvacc[u % DB]);
-        dkacc[u % DB] = Tr::mfma32(cq[u], dsb[bc][u / DB], dkacc[u % DB]);
-      }
-      if (do_v) {
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const int r = 2 * u + e;
-          const float p = __builtin_amdgcn_exp2f(fmaf(s[bv][r], qk_scale, -colc));
-          const float ds = p * dp[bv][r];
-          s[bv][r] = p;
-          dp[bv][r] = ds;
-          csum += ds;
-        }
-        if (u % 4 == 3) {  // eight scores complete: pack one MFMA operand each of P and dS
-          pb[bv][u / 4] = pack8<Tr>(s[bv], 8 * (u / 4));
-          dsb[bv][u / 4] = pack8<Tr>(dp[bv], 8 * (u / 4));
-        }
-      }
-      constexpr int kMfmaMask = 0x008, kValuMask = 0x002, kTransMask = 0x400;
-      const int n_mfma = ((do_s && u < KK) ? 2 : 0) + ((do_c && u < 2 * DB) ? 2 : 0);
-      if (do_v && n_mfma == 4) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(kValuMask, 4, 0);
-          __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
-        }
-      } else if (do_v && n_mfma == 2) {
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-          __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(kValuMask, 8, 0);
-          __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
+    if constexpr (c < NC && slot >= 1 && u < 2 * DB) {
+      cdo[c] = lds_col_operand<D>(do_tile, 32 * bc + 16 * (u / DB), u % DB, lane);
+      cq[c] = lds_col_operand<D>(q_tile, 32 * bc + 16 * (u / DB), u % DB, lane);
     }
-  }
+  };
+  // the accumulators of block b start from the row terms instead of zero; requested PF chunks early too
+  auto init_block = [&](int b) {  // b is a constant at every call site
+    if (b < MB) {
+      s[b] = acc_init(rc_s, 32 * b, g);
+      dp[b] = acc_init(dl_s, 32 * b, g);
+    }
+  };
+  init_block(0);
+  static_for<0, PF>([&](auto ic) { fetch(ic); });
+  static_for<0, NC>([&](auto ic) {
+    constexpr int c = decltype(ic)::value;
+    constexpr int slot = c / NCH - 1, u = c % NCH;
+    constexpr bool do_s = slot + 1 < MB, do_v = slot >= 0 && slot < MB, do_c = slot >= 1;
+    constexpr int bs = slot + 1, bv = slot, bc = slot - 1;
+    fetch(std::integral_constant<int, c + PF>{});
+    if constexpr (u == NCH - PF) init_block(bs + 1);
+    if constexpr (do_s && u < KK) {
+      s[bs] = Tr::mfma32(aq[c], kreg[u], s[bs]);
+      dp[bs] = Tr::mfma32(ado[c], vreg[u], dp[bs]);
+    }
+    if constexpr (do_c && u < 2 * DB) {
+      dvacc[u % DB] = Tr::mfma32(cdo[c], pb[bc][u / DB], dvacc[u % DB]);
+      dkacc[u % DB] = Tr::mfma32(cq[c], dsb[bc][u / DB], dkacc[u % DB]);
+    }
+    if constexpr (do_v) {
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int r = 2 * u + e;
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[bv][r], qk_scale, -colc));
+        const float ds = p * dp[bv][r];
+        s[bv][r] = p;
+        dp[bv][r] = ds;
+        csum += ds;
+      }
+      if constexpr (u % 4 == 3) {  // eight scores complete: pack one MFMA operand each of P and dS
+        pb[bv][u / 4] = pack8<Tr>(s[bv], 8 * (u / 4));
+        dsb[bv][u / 4] = pack8<Tr>(dp[bv], 8 * (u / 4));
+      }
+    }
+    constexpr int kMfmaMask = 0x008, kValuMask = 0x002, kTransMask = 0x400;
+    constexpr int n_mfma = ((do_s && u < KK) ? 2 : 0) + ((do_c && u < 2 * DB) ? 2 : 0);
+    if constexpr (do_v && n_mfma == 4) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(kValuMask, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
+      }
+    } else if constexpr (do_v && n_mfma == 2) {
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(kValuMask, 8, 0);
+        __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  });
 }
 
 template <typename Tr, int D>

@@ -6,7 +6,21 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+#include <utility>
+
 namespace fox {
+
+// Compile-time loop: f(std::integral_constant<int, I>{}) for I = BEGIN .. END-1, so that everything
+// derived from the index is a constant expression inside f.
+template <int BEGIN, typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, BEGIN + I>{}), ...);
+}
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl<BEGIN>(f, std::make_integer_sequence<int, END - BEGIN>{});
+}
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
