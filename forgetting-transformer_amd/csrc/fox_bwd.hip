@@ -101,8 +101,8 @@ __device__ __forceinline__ void dkdv_step(const char* q_tile, const char* do_til
 //   * the vector arithmetic  P, dS   of block b,
 //   * the accumulation MFMAs dV, dK  of block b-1,
 // which are mutually independent.  A scheduling fence after every chunk keeps the
-// compiler from regrouping them; the LDS operands of a chunk are requested two
-// chunks (about eight MFMAs) ahead, across slot boundaries, so their latency hides
+// compiler from regrouping them; the LDS operands of a chunk are requested four
+// chunks (about sixteen MFMAs) ahead, across slot boundaries, so their latency hides
 // behind the chunks in between.
 template <typename Tr, int D>
 __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
@@ -111,7 +111,7 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
                                           float qk_scale, float colc, int lane) {
   constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32, NCH = 8;
   constexpr int NC = (MB + 2) * NCH;  // chunks of the step: slots -1 .. MB
-  constexpr int PF = 2;               // LDS operands are requested this many chunks before their MFMAs
+  constexpr int PF = 4;               // LDS operands are requested this many chunks before their MFMAs
   static_assert(KK <= NCH && 2 * DB <= NCH, "one k-step and one accumulation pair per chunk");
   const int g = lane >> 5, i = lane & 31;
   f32x16 s[MB], dp[MB];
