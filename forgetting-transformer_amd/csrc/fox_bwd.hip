@@ -228,16 +228,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   // query range: rows whose key position reaches this tile, up to the pruning bound
   int m_lo = max(n0 - p_seq, 0);
   m_lo = (m_lo / BMQ) * BMQ;
-  int m_hi = M;
-  if (a.thr) {
-    const int last = min(N - 1, n0 + BN - 1);
-    const int U = (M + BMQ - 1) / BMQ;
-    const int u = acp_first_pruned_qblock(c_row, c_row[last], a.thr[bh], p_seq, BMQ, m_lo / BMQ, U, lane);
-    m_hi = min(M, u * BMQ);
-  }
-  if (n0 + BN <= seq) m_hi = m_lo;  // every key of the tile is left padding
-  const int n_steps = m_hi > m_lo ? (m_hi - m_lo + BMQ - 1) / BMQ : 0;
-
   const int n_w0 = n0 + 32 * wave;
   const int n = n_w0 + i;  // this lane's key row
   u32x4 kreg[KK], vreg[KK];
@@ -266,6 +256,21 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     qld.issue(qp, a.q.st, ms, M, qt);
     dold.issue(dop, a.d_o.st, ms, M, dot);
   };
+  // The first diagonal step does not depend on the pruning bound: its tile is requested before the
+  // bound search, whose own loads then wait behind it once.
+  const bool early = m_lo < M && p_seq + m_lo < n0 + BN - 1 && !(n0 + BN <= seq);
+  if (early) issue(m_lo, q_tile1, do_tile1);
+
+  int m_hi = M;
+  if (a.thr) {
+    const int last = min(N - 1, n0 + BN - 1);
+    const int U = (M + BMQ - 1) / BMQ;
+    const int u = acp_first_pruned_qblock(c_row, c_row[last], a.thr[bh], p_seq, BMQ, m_lo / BMQ, U, lane);
+    m_hi = min(M, u * BMQ);
+  }
+  if (n0 + BN <= seq) m_hi = m_lo;  // every key of the tile is left padding
+  const int n_steps = m_hi > m_lo ? (m_hi - m_lo + BMQ - 1) / BMQ : 0;
+
   // Phase 1: the steps that touch the tile's diagonal (at most BN/BMQ + 1 of them) run one at a
   // time through buffer 1 with the masking code; the first interior tile is requested into
   // buffer 0 before the last of them is computed.  Phase 2: interior steps, double-buffered,
@@ -277,8 +282,10 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   const int n_int = n_steps - n_diag, m_top = m_lo + (n_steps - 1) * BMQ;
   for (int t = 0; t < n_diag; ++t) {
     const int ms = m_lo + t * BMQ;
-    __syncthreads();  // buffer 1 is free again
-    issue(ms, q_tile1, do_tile1);
+    if (!(early && t == 0)) {
+      __syncthreads();  // buffer 1 is free again
+      issue(ms, q_tile1, do_tile1);
+    }
     if (tid < BMQ) { rc_s1[tid] = rc_pref; dl_s1[tid] = dl_pref; }
     wait_vmem_all();
     __syncthreads();
@@ -303,6 +310,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     if (t + 2 < n_int && tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
   }
 
+  if (early && n_steps == 0) wait_vmem_all();  // the requested tile must land before the workgroup's LDS is released
   const float ctot = half_sum(csum);
   if (n < N) {
 #pragma unroll
@@ -397,14 +405,6 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     const int64_t s64 = a.seq_start[b];
     seq = (int)(s64 < 0 ? 0 : (s64 > N ? N : s64));
   }
-  int lo = min(seq, hi);
-  if (a.thr) {
-    const int t = acp_first_kept_block(c_row, c_row[a0], a.thr[bh], N, BN, a0 / BN, lane);
-    lo = max(lo, t * BN);
-  }
-  lo = (lo / BN) * BN;
-  const int n_tiles = (hi - lo + BN - 1) / BN;
-
   const int m = m0 + 32 * wave + i;
   const int a_m = p_seq + m;
   const int a_w0 = a0 + 32 * wave;
@@ -438,6 +438,20 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     kld.issue(kp, a.k.st, n0, N, kt);
     vld.issue(vp, a.v.st, n0, N, vt);
   };
+  // The first tile to visit does not depend on the pruning bound: its loads are requested before the
+  // bound search, whose own loads then wait behind them once.
+  const int n0_first = hi > 0 ? ((hi - 1) / BN) * BN : 0;
+  const bool early = hi > (min(seq, hi) / BN) * BN;
+  if (early) issue(n0_first, k_tile0, v_tile0);
+
+  int lo = min(seq, hi);
+  if (a.thr) {
+    const int t = acp_first_kept_block(c_row, c_ref, a.thr[bh], N, BN, a0 / BN, lane);
+    lo = max(lo, t * BN);
+  }
+  lo = (lo / BN) * BN;
+  const int n_tiles = (hi - lo + BN - 1) / BN;
+
   const bool wave_has_rows = m0 + 32 * wave < M;  // a wave without query rows only moves tiles
   auto compute = [&](int n0, const char* kt, const char* vt, const float* cn) {
     if (!wave_has_rows) return;
@@ -445,7 +459,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
   };
 
   if (n_tiles > 0) {
-    issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
+    if (!early) issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
     if (tid < BN) cn_s0[tid] = cn_pref;
   }
   for (int t = n_tiles - 1; t >= 0; t -= 2) {

@@ -238,21 +238,6 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     const int64_t s64 = a.seq_start[b];
     seq = (int)(s64 < 0 ? 0 : (s64 > N ? N : s64));
   }
-  int lo = min(seq, hi);
-  if (a.thr) {
-    const int t = acp_first_kept_block(c_row, c_row[a0], a.thr[bh], N, BN, a0 / BN, lane);
-    lo = max(lo, t * BN);
-  }
-  lo = (lo / BN) * BN;
-  if (a.first_block && tid == 0 && sp == 0) a.first_block[(int64_t)bh * a.n_mtiles + mt] = lo / BN;
-  int n_tiles = (hi - lo + BN - 1) / BN;  // walked from the last (diagonal) tile down to lo
-  if constexpr (SPLIT) {  // this workgroup's contiguous share of the key tiles
-    const int per = (n_tiles + a.splits - 1) / a.splits;
-    const int t0 = min(n_tiles, sp * per), t1 = min(n_tiles, t0 + per);
-    lo += t0 * BN;
-    n_tiles = t1 - t0;
-  }
-
   const int m = m0 + 32 * wave + i;  // this lane's query row
   const int a_m = p_seq + m;
   const int a_w0 = a0 + 32 * wave;   // key position of the wave's first row
@@ -280,6 +265,28 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     kld.issue(kp, a.k.st, n0, N, kt);
     vld.issue(vp, a.v.st, n0, N, vt);
   };
+  // The first tile to visit (the one under the end of the diagonal) does not depend on the pruning
+  // bound, so its loads are requested before the bound search: the search's own loads then wait
+  // behind them once, instead of three memory latencies in a row.
+  const int n0_first = hi > 0 ? ((hi - 1) / BN) * BN : 0;
+  const bool early = !SPLIT && hi > (min(seq, hi) / BN) * BN && (n0_first + BN - 1 > a0 || !(qk_scale > 0.f));
+  if (early) issue(n0_first, k_tile0, v_tile0);
+
+  int lo = min(seq, hi);
+  if (a.thr) {
+    const int t = acp_first_kept_block(c_row, c_ref, a.thr[bh], N, BN, a0 / BN, lane);
+    lo = max(lo, t * BN);
+  }
+  lo = (lo / BN) * BN;
+  if (a.first_block && tid == 0 && sp == 0) a.first_block[(int64_t)bh * a.n_mtiles + mt] = lo / BN;
+  int n_tiles = (hi - lo + BN - 1) / BN;  // walked from the last (diagonal) tile down to lo
+  if constexpr (SPLIT) {  // this workgroup's contiguous share of the key tiles
+    const int per = (n_tiles + a.splits - 1) / a.splits;
+    const int t0 = min(n_tiles, sp * per), t1 = min(n_tiles, t0 + per);
+    lo += t0 * BN;
+    n_tiles = t1 - t0;
+  }
+
   // A wave whose 32 rows all lie beyond M (decode and other short query blocks) still moves its share
   // of every tile but computes nothing.
   const bool wave_has_rows = m0 + 32 * wave < M;
@@ -297,7 +304,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   if (!(qk_scale > 0.f)) n_diag = n_tiles;
   const int t_stop = n_tiles - n_diag;
   if (n_diag > 0) {
-    issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
+    if (!early) issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
     if (tid < BN) cn_s0[tid] = cn_pref;
   }
   for (int t = n_tiles - 1; t >= t_stop; t -= 2) {
