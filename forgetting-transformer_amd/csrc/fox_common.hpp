@@ -283,20 +283,29 @@ __device__ __forceinline__ void decode_block(int wid, int n_tiles, int n_bh, int
 // Adaptive Computation Pruning, query-side bound: the first key block of width BN
 // in [0, t_max] whose largest decay  c_out - c[last column of the block]  is not
 // below thr.  c is non-increasing, so the blocks before it are exactly the
-// prunable ones.  Evaluated by all 64 lanes at once; the result is wave-uniform.
+// prunable ones and the kept blocks form one run that ends at t_max.  The search
+// walks back from t_max, 64 candidate blocks per round (one per lane, one memory
+// round trip): where pruning bites, the run is short and the first round finds its
+// start; where nothing is pruned the rounds are few against the work that follows.
+// Evaluated by all 64 lanes at once; the result is wave-uniform.  Returns t_max when
+// no block qualifies (the diagonal block is always visited).
 __device__ __forceinline__ int acp_first_kept_block(const float* c_row, float c_out, float thr, int N, int BN, int t_max, int lane) {
-  for (int base = 0; base <= t_max; base += kWave) {
-    const int t = base + lane;
+  int first = t_max;
+  for (int top = t_max; top >= 0; top -= kWave) {
+    const int t = top - lane;
     bool keep = false;
-    if (t <= t_max) {
+    if (t >= 0) {
       int col = t * BN + BN - 1;
       col = col < N - 1 ? col : N - 1;
       keep = !((c_out - c_row[col]) < thr);
     }
     const unsigned long long m = __ballot(keep);
-    if (m) return base + __ffsll((long long)m) - 1;
+    if (m == 0) break;                                  // the run ended exactly at the previous round
+    first = top - (63 - __clzll((long long)m));          // lowest kept block of this round
+    const int valid = top + 1 < kWave ? top + 1 : kWave;
+    if (__popcll(m) < valid) break;                     // a pruned block inside this round: the run starts here
   }
-  return t_max;
+  return first;
 }
 
 // Key-side bound: the first query block (BMQ rows, first row u*BMQ) in [u_lo, U)
