@@ -106,8 +106,9 @@ def event_time(fn, iters, warmup=2):
     return start.elapsed_time(end) * 1e-3 / iters
 
 
-def stage_times(w, tensors, iters):
-    """Time every kernel of the path alone through the C ABI (launches go to torch's current stream)."""
+def stage_times(w, tensors, iters, threshold=None):
+    """Time every kernel of the path alone through the C ABI (launches go to torch's current stream).
+    threshold: optional pruning threshold (a float) applied to every (batch, head)."""
     from forgetting_transformer.ops import _lib
     from forgetting_transformer.ops.forgetting_attention import _view
 
@@ -128,7 +129,11 @@ def stage_times(w, tensors, iters):
     ws_bytes = C.c_int64(0)
     _lib.check(lib.fox_attn_fwd_workspace_bytes(C.byref(dims), C.byref(ws_bytes)), "workspace")
     ws = torch.empty(max(ws_bytes.value, 16), dtype=torch.uint8, device=dev)  # key-split partials (prefill / decode shapes)
-    fwd = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), c.data_ptr(), lse.data_ptr(), ss, None,
+    thr = None
+    if threshold is not None:
+        thr_t = torch.full((B, H), float(threshold), dtype=torch.float32, device=dev)
+        thr = thr_t.data_ptr()
+    fwd = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), c.data_ptr(), lse.data_ptr(), ss, thr,
                        1.0 / math.sqrt(D), None, ws.data_ptr() if ws_bytes.value else None, ws_bytes.value)
     out = {}
 
@@ -161,7 +166,7 @@ def stage_times(w, tensors, iters):
     dg = torch.empty_like(c)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     bwd = _lib.BwdArgs(dims, _view(q), _view(k), _view(v), _view(o), _view(dout), _view(dq), _view(dk), _view(dv),
-                       c.data_ptr(), lse.data_ptr(), ss, None, 1.0 / math.sqrt(D), delta.data_ptr(), dc.data_ptr(),
+                       c.data_ptr(), lse.data_ptr(), ss, thr, 1.0 / math.sqrt(D), delta.data_ptr(), dc.data_ptr(),
                        dg.data_ptr())
     for name, fn in (("bwd_delta", lib.fox_attn_bwd_delta), ("bwd_dkdv", lib.fox_attn_bwd_dkdv),
                      ("bwd_dq", lib.fox_attn_bwd_dq)):
@@ -241,6 +246,12 @@ def acp_report(steps, warmup):
             entry.update(pruned_tile_fraction=1.0 - kept, speedup_vs_none=base / t,
                          max_abs_diff_vs_none=(out.float() - ref_out.float()).abs().max().item())
         rep[name] = entry
+    # where the pruned step spends its time: every kernel alone at threshold -10, against the bytes it must move
+    q, k, v, log_fgate = (x.detach() for x in (q, k, v, log_fgate))
+    st = stage_times(w, (q, k, v, log_fgate, dout, None), max(3, steps), threshold=-10.0)
+    S, R = w["B"] * w["H"] * w["M"] * w["D"] * 2, w["B"] * w["H"] * w["M"] * 4
+    alg = {"fwd": 4 * S + 2 * R, "bwd_delta": 2 * S + R, "bwd_dkdv": 6 * S + 4 * R, "bwd_dq": 5 * S + 4 * R}
+    rep["pruned_kernels"] = {k_: {"ms": st[k_] * 1e3, "algorithmic_gbps": alg[k_] / st[k_] * 1e-9} for k_ in alg}
     return rep
 
 
