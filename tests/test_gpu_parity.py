@@ -320,6 +320,44 @@ def test_linearity_in_values_and_upstream_gradient(fa):
 
 
 # --------------------------------------------------------------------------------------
+# seeded sweep over random configurations
+# --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("case", range(48))
+def test_random_configurations(fa, case):
+    """Shapes, layouts, paddings, thresholds and scales drawn from a fixed seed per case: tails of every
+    tile size, M << N, tiny sequences, empty rows, per-head thresholds, both dtypes."""
+    rng = np.random.default_rng(1000 + case)
+    D = int(rng.choice([16, 32, 64, 128]))
+    B, H = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+    N = int(rng.choice([1, 2, 31, 64, 65, 127, 128, 129, 200, 257, 383, 512, 777, 1025]))
+    M = int(rng.choice([1, max(1, N // 3), max(1, N - 1), N]))
+    dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+    head_first = bool(rng.random() < 0.5)
+    seq = None if rng.random() < 0.5 else [int(x) for x in rng.integers(0, N + 1, size=B)]
+    thr_kind = rng.choice(["none", "float", "auto", "per_head"])
+    thr = {"none": None, "float": float(-rng.uniform(0.5, 30.0)), "auto": "auto",
+           "per_head": torch.tensor(-rng.uniform(1.0, 50.0, size=H), dtype=torch.float32, device="cuda")}[str(thr_kind)]
+    sm_scale = None if rng.random() < 0.7 else float(rng.uniform(0.05, 1.5))
+    gate_mean, gate_std = float(rng.uniform(-2.0, 5.0)), float(rng.uniform(0.3, 2.0))
+    q, k, v, g, do, ss = make_inputs(B, H, M, N, D, dtype=dtype, device="cuda", head_first=head_first, seq_start=seq,
+                                     seed=case, gate_mean=gate_mean, gate_std=gate_std, qkv_std=0.7)
+    # the oracle never prunes; a finite threshold may drop mass up to exp(thr) per pruned entry, so thresholds
+    # above -12 are compared with a pruning-aware tolerance
+    ref = O.forgetting_attention_ref_grads(q, k, v, g, do, head_first=head_first, seq_start=ss, sm_scale=sm_scale, bh_chunk=4)
+    q, k, v, g = (x.requires_grad_() for x in (q, k, v, g))
+    out = fa(q, k, v, g, head_first=head_first, seq_start=ss, sm_scale=sm_scale, adaptive_threshold=thr)
+    out.backward(do)
+    loose = thr_kind in ("float", "per_head")
+    tol = REL_TOL if dtype == torch.bfloat16 else 1e-2
+    if loose:
+        worst = float(thr) if thr_kind == "float" else float(thr.max().item())
+        tol = tol + 4.0 * N * math.exp(worst)    # mass a row can lose: at most N entries of weight e^thr (scores are O(1))
+    for name, x, r in zip(("out", "dq", "dk", "dv", "dlog_fgate"), (out, q.grad, k.grad, v.grad, g.grad), ref):
+        assert torch.isfinite(x).all(), (name, case)
+        assert rel_err(x, r) <= tol, (name, case, rel_err(x, r), tol, dict(B=B, H=H, M=M, N=N, D=D, thr=thr_kind))
+
+
+# --------------------------------------------------------------------------------------
 # benchmark configurations 3-5 at full size
 # --------------------------------------------------------------------------------------
 def _full_size_check(fa, B, H, T, D, mean, std, thr, pairs):
