@@ -14,11 +14,13 @@
 
 namespace fox {
 
+constexpr int kScanThreads = 1024;  // one workgroup per row: few rows, long rows, so the workgroup is as wide as it gets
+
 // Scan of one row: element idx is produced by load(idx) and the running sum up to and including
 // it is handed to store(idx, sum).  REVERSE walks the row from its last element to its first.
 template <bool REVERSE, typename Load, typename Store>
 __device__ __forceinline__ void scan_row(int N, Load load, Store store) {
-  constexpr int PER = 8, NT = 256, SPAN = PER * NT;
+  constexpr int PER = 8, NT = kScanThreads, SPAN = PER * NT;
   __shared__ double wave_tot[NT / kWave];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   double carry = 0.0;
@@ -72,7 +74,7 @@ __device__ __forceinline__ void scan_row(int N, Load load, Store store) {
 }
 
 template <bool REVERSE>
-__global__ __launch_bounds__(256) void scan_kernel(const float* __restrict__ in, int64_t sb, int64_t sh, int64_t sn,
+__global__ __launch_bounds__(kScanThreads) void scan_kernel(const float* __restrict__ in, int64_t sb, int64_t sh, int64_t sn,
                                                    const int64_t* __restrict__ seq_start, float* __restrict__ out, int H,
                                                    int N) {
   const int bh = blockIdx.x, b = bh / H, h = bh % H;
@@ -116,7 +118,7 @@ __device__ __forceinline__ float log_sigmoid(float x) {
 // c[n] = sum_{seq_start <= l <= n} logsigmoid(x[l]) in one pass over the logits; optionally also
 // stores log_fgate[n] = logsigmoid(x[n]) (the decode cache of the FoX layer keeps it).
 template <int DT>
-__global__ __launch_bounds__(256) void gate_scan_fwd_kernel(const void* __restrict__ logits, int64_t sb, int64_t sh, int64_t sn,
+__global__ __launch_bounds__(kScanThreads) void gate_scan_fwd_kernel(const void* __restrict__ logits, int64_t sb, int64_t sh, int64_t sn,
                                                             const int64_t* __restrict__ seq_start,
                                                             float* __restrict__ log_fgate, float* __restrict__ out, int H,
                                                             int N) {
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(256) void gate_scan_fwd_kernel(const void* __restri
 // dlogit[l] = (sum_{n>=l} dc[n]) * d logsigmoid(x_l)/dx = dg[l] * (1 - sigmoid(x_l)), stored in the
 // dtype and layout of the logits.
 template <int DT>
-__global__ __launch_bounds__(256) void gate_scan_bwd_kernel(const float* __restrict__ dc, const void* __restrict__ logits,
+__global__ __launch_bounds__(kScanThreads) void gate_scan_bwd_kernel(const float* __restrict__ dc, const void* __restrict__ logits,
                                                             int64_t sb, int64_t sh, int64_t sn, void* __restrict__ dlogits,
                                                             int64_t db, int64_t dh, int64_t dn, int H, int N) {
   const int bh = blockIdx.x, b = bh / H, h = bh % H;
@@ -163,9 +165,9 @@ hipError_t launch_gate_cumsum_fwd(const void* logits, int dtype, int64_t sb, int
                                   float* log_fgate, float* c, int B, int H, int N, hipStream_t s) {
   const dim3 grid((unsigned)(B * H));
   switch (dtype) {
-    case 0: hipLaunchKernelGGL(gate_scan_fwd_kernel<0>, grid, dim3(256), 0, s, logits, sb, sh, sn, seq_start, log_fgate, c, H, N); break;
-    case 1: hipLaunchKernelGGL(gate_scan_fwd_kernel<1>, grid, dim3(256), 0, s, logits, sb, sh, sn, seq_start, log_fgate, c, H, N); break;
-    case 2: hipLaunchKernelGGL(gate_scan_fwd_kernel<2>, grid, dim3(256), 0, s, logits, sb, sh, sn, seq_start, log_fgate, c, H, N); break;
+    case 0: hipLaunchKernelGGL(gate_scan_fwd_kernel<0>, grid, dim3(kScanThreads), 0, s, logits, sb, sh, sn, seq_start, log_fgate, c, H, N); break;
+    case 1: hipLaunchKernelGGL(gate_scan_fwd_kernel<1>, grid, dim3(kScanThreads), 0, s, logits, sb, sh, sn, seq_start, log_fgate, c, H, N); break;
+    case 2: hipLaunchKernelGGL(gate_scan_fwd_kernel<2>, grid, dim3(kScanThreads), 0, s, logits, sb, sh, sn, seq_start, log_fgate, c, H, N); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
@@ -175,9 +177,9 @@ hipError_t launch_gate_cumsum_bwd(const float* dc, const void* logits, int dtype
                                   void* dlogits, int64_t db, int64_t dh, int64_t dn, int B, int H, int N, hipStream_t s) {
   const dim3 grid((unsigned)(B * H));
   switch (dtype) {
-    case 0: hipLaunchKernelGGL(gate_scan_bwd_kernel<0>, grid, dim3(256), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
-    case 1: hipLaunchKernelGGL(gate_scan_bwd_kernel<1>, grid, dim3(256), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
-    case 2: hipLaunchKernelGGL(gate_scan_bwd_kernel<2>, grid, dim3(256), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
+    case 0: hipLaunchKernelGGL(gate_scan_bwd_kernel<0>, grid, dim3(kScanThreads), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
+    case 1: hipLaunchKernelGGL(gate_scan_bwd_kernel<1>, grid, dim3(kScanThreads), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
+    case 2: hipLaunchKernelGGL(gate_scan_bwd_kernel<2>, grid, dim3(kScanThreads), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
@@ -185,12 +187,12 @@ hipError_t launch_gate_cumsum_bwd(const float* dc, const void* logits, int dtype
 
 hipError_t launch_cumsum_fwd(const float* g, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start, float* c, int B,
                              int H, int N, hipStream_t s) {
-  hipLaunchKernelGGL(scan_kernel<false>, dim3((unsigned)(B * H)), dim3(256), 0, s, g, sb, sh, sn, seq_start, c, H, N);
+  hipLaunchKernelGGL(scan_kernel<false>, dim3((unsigned)(B * H)), dim3(kScanThreads), 0, s, g, sb, sh, sn, seq_start, c, H, N);
   return hipGetLastError();
 }
 
 hipError_t launch_cumsum_bwd(const float* dc, float* dg, int B, int H, int N, hipStream_t s) {
-  hipLaunchKernelGGL(scan_kernel<true>, dim3((unsigned)(B * H)), dim3(256), 0, s, dc, (int64_t)H * N, (int64_t)N, (int64_t)1,
+  hipLaunchKernelGGL(scan_kernel<true>, dim3((unsigned)(B * H)), dim3(kScanThreads), 0, s, dc, (int64_t)H * N, (int64_t)N, (int64_t)1,
                      (const int64_t*)nullptr, dg, H, N);
   return hipGetLastError();
 }
