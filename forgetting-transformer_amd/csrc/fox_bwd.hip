@@ -312,24 +312,13 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
 
   if (early && n_steps == 0) wait_vmem_all();  // the requested tile must land before the workgroup's LDS is released
   const float ctot = half_sum(csum);
-  if (n < N) {
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int d = 32 * db + 8 * q4 + 4 * g;
-        if (d < D) {
-          u32x2 w;
-          w[0] = Tr::pack2(dkacc[db][4 * q4 + 0] * a.sm_scale, dkacc[db][4 * q4 + 1] * a.sm_scale);
-          w[1] = Tr::pack2(dkacc[db][4 * q4 + 2] * a.sm_scale, dkacc[db][4 * q4 + 3] * a.sm_scale);
-          *reinterpret_cast<u32x2*>(dkp + (int64_t)n * a.dk.st + d) = w;
-          w[0] = Tr::pack2(dvacc[db][4 * q4 + 0], dvacc[db][4 * q4 + 1]);
-          w[1] = Tr::pack2(dvacc[db][4 * q4 + 2], dvacc[db][4 * q4 + 3]);
-          *reinterpret_cast<u32x2*>(dvp + (int64_t)n * a.dv.st + d) = w;
-        }
-      }
-    if (g == 0) a.dc[(int64_t)bh * N + n] = -ctot;
-  }
+  if (n < N && g == 0) a.dc[(int64_t)bh * N + n] = -ctot;
+  // dK and dV leave through LDS (the tile buffers are free now) so that the global stores are whole rows
+  static_assert(2 * kStoreStageBytes<D> <= Tile<D>::bytes(BMQ), "two waves stage in one tile buffer");
+  __syncthreads();  // every wave is done with the tiles of the last step
+  char* stage = (wave < 2 ? q_tile0 : do_tile0) + (wave & 1) * kStoreStageBytes<D>;
+  store_rows_via_lds<Tr, D>(stage, dkacc, a.sm_scale, dkp, a.dk.st, n_w0, N, lane);
+  store_rows_via_lds<Tr, D>(stage, dvacc, 1.0f, dvp, a.dv.st, n_w0, N, lane);
 }
 
 // ---------------------------------------------------------------------------

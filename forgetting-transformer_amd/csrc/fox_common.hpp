@@ -246,6 +246,46 @@ __device__ __forceinline__ float half_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Store a wave's transposed accumulator block as rows of 16-bit values.  Lane (g, i) holds row i of
+// 32 rows; register r of acc[db] is column 32*db + 8*(r/4) + 4*g + r%4.  Written straight to global
+// memory that is 8 bytes per lane scattered over 32 rows; staged through a wave-private LDS area of
+// kStoreStageBytes<D> the global stores are 16 bytes per lane and each instruction covers whole rows.
+// Rows at or beyond row_limit are not stored.  The caller makes sure nobody else uses the staging area.
+template <int D>
+constexpr int kStoreStageBytes = 32 * (2 * D + 16);
+
+template <typename Tr, int D>
+__device__ __forceinline__ void store_rows_via_lds(char* stage, const f32x16 (&acc)[(D + 31) / 32], float mul, uint16_t* dst,
+                                                   int64_t row_stride, int row0, int row_limit, int lane) {
+  constexpr int DB = (D + 31) / 32, CH = D / 8, RS = 2 * D + 16;
+  const int g = lane >> 5, i = lane & 31;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const int d = 32 * db + 8 * q4 + 4 * g;
+      if (d < D) {
+        u32x2 w;
+        w[0] = Tr::pack2(acc[db][4 * q4 + 0] * mul, acc[db][4 * q4 + 1] * mul);
+        w[1] = Tr::pack2(acc[db][4 * q4 + 2] * mul, acc[db][4 * q4 + 3] * mul);
+        *reinterpret_cast<u32x2*>(stage + i * RS + 2 * d) = w;
+      }
+    }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int idx0 = 0; idx0 < 32 * CH; idx0 += kWave) {
+    const int idx = idx0 + lane, row = idx / CH, ch = idx % CH;
+    if ((32 * CH % kWave == 0 || idx < 32 * CH) && row0 + row < row_limit) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * RS + 16 * ch);
+      *reinterpret_cast<u32x4*>(dst + (int64_t)(row0 + row) * row_stride + 8 * ch) = v;
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();   // the staging area may be rewritten after this
+}
+
 // Start value of a 32x32 MFMA accumulator whose row r carries the per-row term
 // t[row0 + r] (read from LDS): the matrix pipe then adds the dot products to it for
 // free, which saves one vector instruction per score.
