@@ -466,21 +466,12 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
   }
 
   const float rtot = half_sum(rsum);
-  if (m < M) {
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int d = 32 * db + 8 * q4 + 4 * g;
-        if (d < D) {
-          u32x2 w;
-          w[0] = Tr::pack2(dqacc[db][4 * q4 + 0] * a.sm_scale, dqacc[db][4 * q4 + 1] * a.sm_scale);
-          w[1] = Tr::pack2(dqacc[db][4 * q4 + 2] * a.sm_scale, dqacc[db][4 * q4 + 3] * a.sm_scale);
-          *reinterpret_cast<u32x2*>(dqp + (int64_t)m * a.dq.st + d) = w;
-        }
-      }
-    if (g == 0) a.dc[(int64_t)bh * N + a_m] += rtot;  // the dK/dV kernel wrote the column part earlier on this stream
-  }
+  if (m < M && g == 0) a.dc[(int64_t)bh * N + a_m] += rtot;  // the dK/dV kernel wrote the column part earlier on this stream
+  // dQ leaves through LDS (the tile buffers are free now, one per wave) so that the global stores are whole rows
+  static_assert(kStoreStageBytes<D> <= Tile<D>::bytes(BN), "one wave stages in one tile buffer");
+  __syncthreads();  // every wave is done with the last tile
+  char* stage = wave == 0 ? k_tile0 : wave == 1 ? k_tile1 : wave == 2 ? v_tile0 : v_tile1;
+  store_rows_via_lds<Tr, D>(stage, dqacc, a.sm_scale, dqp, a.dq.st, m0 + 32 * wave, M, lane);
 }
 
 // explicit instantiations: every (dtype, head dim) pair the dispatchers can reach

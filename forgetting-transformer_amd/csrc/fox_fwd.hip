@@ -398,21 +398,12 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   }
   const bool empty = a_m < seq;
   const float inv = empty ? 0.f : 1.0f / l_tot;
-  if (m < M) {
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        const int d = 32 * db + 8 * q4 + 4 * g;
-        if (d < D) {
-          u32x2 w;
-          w[0] = Tr::pack2(oacc[db][4 * q4 + 0] * inv, oacc[db][4 * q4 + 1] * inv);
-          w[1] = Tr::pack2(oacc[db][4 * q4 + 2] * inv, oacc[db][4 * q4 + 3] * inv);
-          *reinterpret_cast<u32x2*>(op + (int64_t)m * a.o.st + d) = w;
-        }
-      }
-    if (g == 0) a.lse[(int64_t)bh * M + m] = empty ? -INFINITY : (m_i + cm2) * kLn2 + __logf(l_tot);
-  }
+  if (m < M && g == 0) a.lse[(int64_t)bh * M + m] = empty ? -INFINITY : (m_i + cm2) * kLn2 + __logf(l_tot);
+  // o leaves through LDS (the tile buffers are free now, one per wave) so that the global stores are whole rows
+  static_assert(kStoreStageBytes<D> <= Tile<D>::bytes(BN), "one wave stages in one tile buffer");
+  __syncthreads();  // every wave is done with the last tile
+  char* stage = wave == 0 ? k_tile0 : wave == 1 ? k_tile1 : wave == 2 ? v_tile0 : v_tile1;
+  store_rows_via_lds<Tr, D>(stage, oacc, inv, op, a.o.st, m0 + 32 * wave, M, lane);
 }
 
 // Merge the partial results of the key splits of one query row:
