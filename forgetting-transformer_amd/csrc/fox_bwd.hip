@@ -230,12 +230,40 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   m_lo = (m_lo / BMQ) * BMQ;
   const int n_w0 = n0 + 32 * wave;
   const int n = n_w0 + i;  // this lane's key row
+  // Everything the workgroup needs first is requested before anything is waited for: the tile of the
+  // first diagonal step (it does not depend on the pruning bound), K and V, then the per-row terms.
+  const DirectTileLoader<D, BMQ> qld(a.q.st, wave, lane), dold(a.d_o.st, wave, lane);
+  const bool early = m_lo < M && p_seq + m_lo < n0 + BN - 1 && !(n0 + BN <= seq);
+  if (early) {
+    qld.issue(qp, a.q.st, m_lo, M, q_tile1);
+    dold.issue(dop, a.d_o.st, m_lo, M, do_tile1);
+  }
   u32x4 kreg[KK], vreg[KK];
   load_row_operand_regs<D>(kreg, kp, a.k.st, n, N, g);
   load_row_operand_regs<D>(vreg, vp, a.v.st, n, N, g);
   const float c_ref = c_row[n0];
-  const float colc = (n < N && n >= seq) ? (c_row[n] - c_ref) * kLog2e : INFINITY;
+  const float c_key = c_row[min(n, N - 1)];
+  const float c_last = c_row[min(N - 1, n0 + BN - 1)];  // for the pruning bound below
   const float qk_scale = nonzero_scale(a.sm_scale * kLog2e), inv_scale = 1.0f / qk_scale;
+
+  float rc_pref = 0.f, dl_pref = 0.f;
+  auto issue_rows = [&](int ms) {  // per-row terms of a step: branch-free loads
+    if (tid < BMQ) {
+      const int mm = ms + tid, mc = min(mm, M - 1);
+      const float l = lse_row[mc], cv = c_row[p_seq + mc], dv = delta_row[mc];
+      // rows past M and empty rows (lse = -inf) get -inf through the subtraction, so that no load hides behind a branch
+      const float l_eff = ((mm < M) & (l > -INFINITY)) ? l : INFINITY;
+      rc_pref = (cv - c_ref - l_eff) * kLog2e * inv_scale;
+      dl_pref = mm < M ? -dv : 0.f;
+    }
+  };
+  auto issue = [&](int ms, char* qt, char* dot) {
+    issue_rows(ms);  // small loads first: vmcnt retires in order, so they must not queue behind the tile
+    qld.issue(qp, a.q.st, ms, M, qt);
+    dold.issue(dop, a.d_o.st, ms, M, dot);
+  };
+  if (early) issue_rows(m_lo);
+  const float colc = (n < N && n >= seq) ? (c_key - c_ref) * kLog2e : INFINITY;
 
   f32x16 dkacc[DB], dvacc[DB];
 #pragma unroll
@@ -244,28 +272,11 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
   float csum = 0.f;
 
-  const DirectTileLoader<D, BMQ> qld(a.q.st, wave, lane), dold(a.d_o.st, wave, lane);
-  float rc_pref = 0.f, dl_pref = 0.f;
-  auto issue = [&](int ms, char* qt, char* dot) {
-    if (tid < BMQ) {  // small loads first and branch-free: vmcnt retires in order
-      const int mm = ms + tid, mc = min(mm, M - 1);
-      const float l = lse_row[mc], cv = c_row[p_seq + mc], dv = delta_row[mc];
-      rc_pref = (mm < M && l > -INFINITY) ? (cv - c_ref - l) * kLog2e * inv_scale : -INFINITY * inv_scale;
-      dl_pref = mm < M ? -dv : 0.f;
-    }
-    qld.issue(qp, a.q.st, ms, M, qt);
-    dold.issue(dop, a.d_o.st, ms, M, dot);
-  };
-  // The first diagonal step does not depend on the pruning bound: its tile is requested before the
-  // bound search, whose own loads then wait behind it once.
-  const bool early = m_lo < M && p_seq + m_lo < n0 + BN - 1 && !(n0 + BN <= seq);
-  if (early) issue(m_lo, q_tile1, do_tile1);
 
   int m_hi = M;
   if (a.thr) {
-    const int last = min(N - 1, n0 + BN - 1);
     const int U = (M + BMQ - 1) / BMQ;
-    const int u = acp_first_pruned_qblock(c_row, c_row[last], a.thr[bh], p_seq, BMQ, m_lo / BMQ, U, lane);
+    const int u = acp_first_pruned_qblock(c_row, c_last, a.thr[bh], p_seq, BMQ, m_lo / BMQ, U, lane);
     m_hi = min(M, u * BMQ);
   }
   if (n0 + BN <= seq) m_hi = m_lo;  // every key of the tile is left padding
@@ -397,17 +408,26 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
   const int m = m0 + 32 * wave + i;
   const int a_m = p_seq + m;
   const int a_w0 = a0 + 32 * wave;
+  const float qk_scale = nonzero_scale(a.sm_scale * kLog2e), inv_scale = 1.0f / qk_scale;
+  // Everything the workgroup needs first is requested before anything is waited for: the first tile to
+  // visit (it does not depend on the pruning bound), Q and dO, then the per-row and per-key terms.
+  const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
+  const int n0_first = hi > 0 ? ((hi - 1) / BN) * BN : 0;
+  const bool early = hi > (min(seq, hi) / BN) * BN;
+  if (early) {
+    kld.issue(kp, a.k.st, n0_first, N, k_tile0);
+    vld.issue(vp, a.v.st, n0_first, N, v_tile0);
+  }
   u32x4 qreg[KK], doreg[KK];
   load_row_operand_regs<D>(qreg, qp, a.q.st, m, M, g);
   load_row_operand_regs<D>(doreg, dop, a.d_o.st, m, M, g);
   const float c_ref = c_row[a0];
-  float rowc = -INFINITY, delta = 0.f;
-  if (m < M) {
-    const float l = a.lse[(int64_t)bh * M + m];
-    if (l > -INFINITY) rowc = (c_row[a_m] - c_ref - l) * kLog2e;
-    delta = a.delta[(int64_t)bh * M + m];
-  }
-  const float qk_scale = nonzero_scale(a.sm_scale * kLog2e), inv_scale = 1.0f / qk_scale;
+  // rows past M and empty rows (lse = -inf) get rowc = -inf through the subtraction: no load behind a branch
+  const int mc = min(m, M - 1);
+  const float l = a.lse[(int64_t)bh * M + mc], c_m = c_row[min(p_seq + mc, N - 1)], dlt = a.delta[(int64_t)bh * M + mc];
+  const float l_eff = ((m < M) & (l > -INFINITY)) ? l : INFINITY;
+  const float rowc = (c_m - c_ref - l_eff) * kLog2e;
+  const float delta = m < M ? dlt : 0.f;
 
   f32x16 dqacc[DB];
 #pragma unroll
@@ -416,22 +436,21 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
   float rsum = 0.f;
 
-  const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
   float cn_pref = 0.f;
-  auto issue = [&](int n0, char* kt, char* vt) {
-    if (tid < BN) {  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
+  auto issue_cn = [&](int n0) {  // key terms of a tile; masked keys get -inf through the subtraction
+    if (tid < BN) {
       const int nn = n0 + tid;
       const float cv = c_row[min(nn, N - 1)];
-      cn_pref = (nn < N && nn >= seq) ? (c_ref - cv) * kLog2e * inv_scale : -INFINITY * inv_scale;
+      const float cv_eff = ((nn < N) & (nn >= seq)) ? cv : INFINITY;
+      cn_pref = (c_ref - cv_eff) * kLog2e * inv_scale;
     }
+  };
+  auto issue = [&](int n0, char* kt, char* vt) {
+    issue_cn(n0);  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
     kld.issue(kp, a.k.st, n0, N, kt);
     vld.issue(vp, a.v.st, n0, N, vt);
   };
-  // The first tile to visit does not depend on the pruning bound: its loads are requested before the
-  // bound search, whose own loads then wait behind them once.
-  const int n0_first = hi > 0 ? ((hi - 1) / BN) * BN : 0;
-  const bool early = hi > (min(seq, hi) / BN) * BN;
-  if (early) issue(n0_first, k_tile0, v_tile0);
+  if (early) issue_cn(n0_first);
 
   int lo = min(seq, hi);
   if (a.thr) {

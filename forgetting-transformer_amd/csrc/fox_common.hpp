@@ -223,12 +223,15 @@ struct DirectTileLoader {
 template <int D>
 __device__ __forceinline__ void load_row_operand_regs(u32x4 (&dst)[D / 16], const uint16_t* base, int64_t row_stride, int row,
                                              int row_limit, int g) {
+  // branch-free: every load is issued before any of them is waited for (rows past the limit read the
+  // last valid row and are zeroed afterwards; row_limit >= 1)
+  const bool valid = row < row_limit;
+  const uint16_t* p = base + (int64_t)(valid ? row : row_limit - 1) * row_stride + 8 * g;
 #pragma unroll
-  for (int kk = 0; kk < D / 16; ++kk) {
-    u32x4 z = {0u, 0u, 0u, 0u};
-    dst[kk] = z;
-    if (row < row_limit) dst[kk] = *reinterpret_cast<const u32x4*>(base + (int64_t)row * row_stride + 16 * kk + 8 * g);
-  }
+  for (int kk = 0; kk < D / 16; ++kk) dst[kk] = *reinterpret_cast<const u32x4*>(p + 16 * kk);
+  const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int kk = 0; kk < D / 16; ++kk) dst[kk] = valid ? dst[kk] : z;
 }
 
 // ---------------------------------------------------------------------------

@@ -241,11 +241,38 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   const int m = m0 + 32 * wave + i;  // this lane's query row
   const int a_m = p_seq + m;
   const int a_w0 = a0 + 32 * wave;   // key position of the wave's first row
+  const float qk_scale = nonzero_scale(a.sm_scale * kLog2e), inv_scale = 1.0f / qk_scale;
+  // Everything the workgroup needs first is requested before anything is waited for.  The first tile to
+  // visit (the one under the end of the diagonal) does not depend on the pruning bound, so it goes
+  // first; then Q, then the per-row and per-key terms; the bound search's loads queue behind them.
+  const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
+  const int n0_first = hi > 0 ? ((hi - 1) / BN) * BN : 0;
+  const bool early = !SPLIT && hi > (min(seq, hi) / BN) * BN && (n0_first + BN - 1 > a0 || !(qk_scale > 0.f));
+  if (early) {
+    kld.issue(kp, a.k.st, n0_first, N, k_tile0);
+    vld.issue(vp, a.v.st, n0_first, N, v_tile0);
+  }
   u32x4 qreg[KK];
   load_row_operand_regs<D>(qreg, qp, a.q.st, m, M, g);
   const float c_ref = c_row[a0];
-  const float cm2 = (m < M) ? (c_row[a_m] - c_ref) * kLog2e : 0.f;
-  const float qk_scale = nonzero_scale(a.sm_scale * kLog2e), inv_scale = 1.0f / qk_scale;
+  const float c_m = c_row[min(a_m, N - 1)];
+
+  float cn_pref = 0.f;
+  auto issue_cn = [&](int n0) {  // key terms of a tile; masked keys get -inf through the subtraction (no load behind a branch)
+    if (tid < BN) {
+      const int n = n0 + tid;
+      const float cv = c_row[min(n, N - 1)];
+      const float cv_eff = ((n < N) & (n >= seq)) ? cv : INFINITY;
+      cn_pref = (c_ref - cv_eff) * kLog2e * inv_scale;
+    }
+  };
+  auto issue = [&](int n0, char* kt, char* vt) {
+    issue_cn(n0);  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
+    kld.issue(kp, a.k.st, n0, N, kt);
+    vld.issue(vp, a.v.st, n0, N, vt);
+  };
+  if (early) issue_cn(n0_first);
+  const float cm2 = (m < M) ? (c_m - c_ref) * kLog2e : 0.f;
 
   f32x16 oacc[DB];
 #pragma unroll
@@ -253,24 +280,6 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
   float m_i = -3.0e38f, l_i = 0.f;  // finite floor: a row that has seen no valid key yet yields exp2(-inf) = 0
-
-  const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
-  float cn_pref = 0.f;
-  auto issue = [&](int n0, char* kt, char* vt) {
-    if (tid < BN) {  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
-      const int n = n0 + tid;
-      const float cv = c_row[min(n, N - 1)];
-      cn_pref = (n < N && n >= seq) ? (c_ref - cv) * kLog2e * inv_scale : -INFINITY * inv_scale;
-    }
-    kld.issue(kp, a.k.st, n0, N, kt);
-    vld.issue(vp, a.v.st, n0, N, vt);
-  };
-  // The first tile to visit (the one under the end of the diagonal) does not depend on the pruning
-  // bound, so its loads are requested before the bound search: the search's own loads then wait
-  // behind them once, instead of three memory latencies in a row.
-  const int n0_first = hi > 0 ? ((hi - 1) / BN) * BN : 0;
-  const bool early = !SPLIT && hi > (min(seq, hi) / BN) * BN && (n0_first + BN - 1 > a0 || !(qk_scale > 0.f));
-  if (early) issue(n0_first, k_tile0, v_tile0);
 
   int lo = min(seq, hi);
   if (a.thr) {
@@ -327,11 +336,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   if (n_int > 0) {
     auto issue_k = [&](int j, char* kt) {
       const int n0 = lo + (n_int - 1 - j) * BN;
-      if (tid < BN) {
-        const int n = n0 + tid;
-        const float cv = c_row[min(n, N - 1)];
-        cn_pref = (n < N && n >= seq) ? (c_ref - cv) * kLog2e * inv_scale : -INFINITY * inv_scale;
-      }
+      issue_cn(n0);
       kld.issue(kp, a.k.st, n0, N, kt);
     };
     auto issue_v = [&](int j, char* vt) { vld.issue(vp, a.v.st, lo + (n_int - 1 - j) * BN, N, vt); };
