@@ -246,17 +246,25 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   const float c_last = c_row[min(N - 1, n0 + BN - 1)];  // for the pruning bound below
   const float qk_scale = nonzero_scale(a.sm_scale * kLog2e), inv_scale = 1.0f / qk_scale;
 
-  float rc_pref = 0.f, dl_pref = 0.f;
-  auto issue_rows = [&](int ms) {  // per-row terms of a step: branch-free loads
+  // Per-row terms of a step: the loads are requested here, the arithmetic on them is done where the values
+  // go to LDS (a step later), so that nothing waits for the loads in between.  Rows past M and empty rows
+  // (lse = -inf) get -inf through the subtraction.
+  float l_raw = 0.f, c_raw = 0.f, d_raw = 0.f;
+  bool row_ok = false;
+  auto issue_rows = [&](int ms) {
     if (tid < BMQ) {
       const int mm = ms + tid, mc = min(mm, M - 1);
-      const float l = lse_row[mc], cv = c_row[p_seq + mc], dv = delta_row[mc];
-      // rows past M and empty rows (lse = -inf) get -inf through the subtraction, so that no load hides behind a branch
-      const float l_eff = ((mm < M) & (l > -INFINITY)) ? l : INFINITY;
-      rc_pref = (cv - c_ref - l_eff) * kLog2e * inv_scale;
-      dl_pref = mm < M ? -dv : 0.f;
+      row_ok = mm < M;
+      l_raw = lse_row[mc];
+      c_raw = c_row[p_seq + mc];
+      d_raw = delta_row[mc];
     }
   };
+  auto rc_term = [&]() {
+    const float l_eff = (row_ok & (l_raw > -INFINITY)) ? l_raw : INFINITY;
+    return (c_raw - c_ref - l_eff) * kLog2e * inv_scale;
+  };
+  auto dl_term = [&]() { return row_ok ? -d_raw : 0.f; };
   auto issue = [&](int ms, char* qt, char* dot) {
     issue_rows(ms);  // small loads first: vmcnt retires in order, so they must not queue behind the tile
     qld.issue(qp, a.q.st, ms, M, qt);
@@ -297,7 +305,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
       __syncthreads();  // buffer 1 is free again
       issue(ms, q_tile1, do_tile1);
     }
-    if (tid < BMQ) { rc_s1[tid] = rc_pref; dl_s1[tid] = dl_pref; }
+    if (tid < BMQ) { rc_s1[tid] = rc_term(); dl_s1[tid] = dl_term(); }
     wait_vmem_all();
     __syncthreads();
     if (t == n_diag - 1 && n_int > 0) issue(m_top, q_tile0, do_tile0);
@@ -305,7 +313,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   }
   if (n_int > 0) {
     if (n_diag == 0) issue(m_top, q_tile0, do_tile0);
-    if (tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
+    if (tid < BMQ) { rc_s0[tid] = rc_term(); dl_s0[tid] = dl_term(); }
   }
   for (int t = 0; t < n_int; t += 2) {
     wait_vmem_all();
@@ -313,12 +321,12 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     if (t + 1 < n_int) issue(m_top - (t + 1) * BMQ, q_tile1, do_tile1);
     dkdv_step_interior<Tr, D>(q_tile0, do_tile0, rc_s0, dl_s0, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane);
     if (t + 1 >= n_int) break;
-    if (tid < BMQ) { rc_s1[tid] = rc_pref; dl_s1[tid] = dl_pref; }
+    if (tid < BMQ) { rc_s1[tid] = rc_term(); dl_s1[tid] = dl_term(); }
     wait_vmem_all();
     __syncthreads();
     if (t + 2 < n_int) issue(m_top - (t + 2) * BMQ, q_tile0, do_tile0);
     dkdv_step_interior<Tr, D>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane);
-    if (t + 2 < n_int && tid < BMQ) { rc_s0[tid] = rc_pref; dl_s0[tid] = dl_pref; }
+    if (t + 2 < n_int && tid < BMQ) { rc_s0[tid] = rc_term(); dl_s0[tid] = dl_term(); }
   }
 
   if (early && n_steps == 0) wait_vmem_all();  // the requested tile must land before the workgroup's LDS is released
@@ -436,15 +444,19 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
   float rsum = 0.f;
 
-  float cn_pref = 0.f;
-  auto issue_cn = [&](int n0) {  // key terms of a tile; masked keys get -inf through the subtraction
+  // Key terms of a tile: the load is requested here, the arithmetic on it is done where the value goes to
+  // LDS (a tile later), so that nothing waits for the load in between.  Masked keys get -inf through the
+  // subtraction.
+  float cn_raw = 0.f;
+  bool cn_ok = false;
+  auto issue_cn = [&](int n0) {
     if (tid < BN) {
       const int nn = n0 + tid;
-      const float cv = c_row[min(nn, N - 1)];
-      const float cv_eff = ((nn < N) & (nn >= seq)) ? cv : INFINITY;
-      cn_pref = (c_ref - cv_eff) * kLog2e * inv_scale;
+      cn_ok = (nn < N) & (nn >= seq);
+      cn_raw = c_row[min(nn, N - 1)];
     }
   };
+  auto cn_term = [&]() { return (c_ref - (cn_ok ? cn_raw : INFINITY)) * kLog2e * inv_scale; };
   auto issue = [&](int n0, char* kt, char* vt) {
     issue_cn(n0);  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
     kld.issue(kp, a.k.st, n0, N, kt);
@@ -468,7 +480,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
 
   if (n_tiles > 0) {
     if (!early) issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
-    if (tid < BN) cn_s0[tid] = cn_pref;
+    if (tid < BN) cn_s0[tid] = cn_term();
   }
   for (int t = n_tiles - 1; t >= 0; t -= 2) {
     wait_vmem_all();
@@ -476,12 +488,12 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     if (t >= 1) issue(lo + (t - 1) * BN, k_tile1, v_tile1);
     compute(lo + t * BN, k_tile0, v_tile0, cn_s0);
     if (t < 1) break;
-    if (tid < BN) cn_s1[tid] = cn_pref;
+    if (tid < BN) cn_s1[tid] = cn_term();
     wait_vmem_all();
     __syncthreads();
     if (t >= 2) issue(lo + (t - 2) * BN, k_tile0, v_tile0);
     compute(lo + (t - 1) * BN, k_tile1, v_tile1, cn_s1);
-    if (t >= 2 && tid < BN) cn_s0[tid] = cn_pref;
+    if (t >= 2 && tid < BN) cn_s0[tid] = cn_term();
   }
 
   const float rtot = half_sum(rsum);

@@ -257,15 +257,19 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   const float c_ref = c_row[a0];
   const float c_m = c_row[min(a_m, N - 1)];
 
-  float cn_pref = 0.f;
-  auto issue_cn = [&](int n0) {  // key terms of a tile; masked keys get -inf through the subtraction (no load behind a branch)
+  // Key terms of a tile: the load is requested here, the arithmetic on it is done where the value goes to
+  // LDS (a tile later), so that nothing waits for the load in between.  Masked keys get -inf through the
+  // subtraction.
+  float cn_raw = 0.f;
+  bool cn_ok = false;
+  auto issue_cn = [&](int n0) {
     if (tid < BN) {
       const int n = n0 + tid;
-      const float cv = c_row[min(n, N - 1)];
-      const float cv_eff = ((n < N) & (n >= seq)) ? cv : INFINITY;
-      cn_pref = (c_ref - cv_eff) * kLog2e * inv_scale;
+      cn_ok = (n < N) & (n >= seq);
+      cn_raw = c_row[min(n, N - 1)];
     }
   };
+  auto cn_term = [&]() { return (c_ref - (cn_ok ? cn_raw : INFINITY)) * kLog2e * inv_scale; };
   auto issue = [&](int n0, char* kt, char* vt) {
     issue_cn(n0);  // small load first: vmcnt retires in order, so it must not queue behind the tile loads
     kld.issue(kp, a.k.st, n0, N, kt);
@@ -314,7 +318,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   const int t_stop = n_tiles - n_diag;
   if (n_diag > 0) {
     if (!early) issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
-    if (tid < BN) cn_s0[tid] = cn_pref;
+    if (tid < BN) cn_s0[tid] = cn_term();
   }
   for (int t = n_tiles - 1; t >= t_stop; t -= 2) {
     // even step: consume buffers 0, fill buffers 1
@@ -323,13 +327,13 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     if (t - 1 >= t_stop) issue(lo + (t - 1) * BN, k_tile1, v_tile1);
     compute(lo + t * BN, k_tile0, v_tile0, cn_s0);
     if (t - 1 < t_stop) break;
-    if (tid < BN) cn_s1[tid] = cn_pref;
+    if (tid < BN) cn_s1[tid] = cn_term();
     // odd step: consume buffers 1, fill buffers 0
     wait_vmem_all();
     __syncthreads();
     if (t - 2 >= t_stop) issue(lo + (t - 2) * BN, k_tile0, v_tile0);
     compute(lo + (t - 1) * BN, k_tile1, v_tile1, cn_s1);
-    if (t - 2 >= t_stop && tid < BN) cn_s0[tid] = cn_pref;
+    if (t - 2 >= t_stop && tid < BN) cn_s0[tid] = cn_term();
   }
 
   const int n_int = t_stop;  // interior tile j (0 = nearest to the diagonal) starts at key lo + (n_int-1-j)*BN
@@ -343,7 +347,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
     // K runs one tile ahead of V: iteration j computes S(j+1) and P(j) V(j).
     __syncthreads();  // phase 1 is done with every buffer
     issue_k(0, k_tile0);
-    if (tid < BN) cn_s0[tid] = cn_pref;
+    if (tid < BN) cn_s0[tid] = cn_term();
     wait_vmem_all();
     __syncthreads();
     if (n_int > 1) issue_k(1, k_tile1);
@@ -360,7 +364,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
       // even iteration: K(j+1) in k_tile1 with its key terms in cn_s1, V(j) in v_tile0.  The key
       // terms of tile j+1 go to LDS before the barrier: their buffer was last read two iterations ago.
       wait_vmem_all();
-      if (j + 1 < n_int && tid < BN) cn_s1[tid] = cn_pref;
+      if (j + 1 < n_int && tid < BN) cn_s1[tid] = cn_term();
       __syncthreads();
       if (j + 2 < n_int) issue_k(j + 2, k_tile0);
       if (j + 1 < n_int) issue_v(j + 1, v_tile1);
@@ -368,7 +372,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
       if (j + 1 >= n_int) break;
       // odd iteration: K(j+2) in k_tile0 with its key terms in cn_s0, V(j+1) in v_tile1
       wait_vmem_all();
-      if (j + 2 < n_int && tid < BN) cn_s0[tid] = cn_pref;
+      if (j + 2 < n_int && tid < BN) cn_s0[tid] = cn_term();
       __syncthreads();
       if (j + 3 < n_int) issue_k(j + 3, k_tile1);
       if (j + 2 < n_int) issue_v(j + 2, v_tile0);
