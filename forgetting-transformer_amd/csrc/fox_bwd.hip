@@ -100,18 +100,24 @@ __device__ __forceinline__ void dkdv_step(const char* q_tile, const char* do_til
 //   * the score MFMAs        S, dP   of block b+1,
 //   * the vector arithmetic  P, dS   of block b,
 //   * the accumulation MFMAs dV, dK  of block b-1,
-// which are mutually independent.  A scheduling fence after every chunk keeps the
-// compiler from regrouping them; the LDS operands of a chunk are requested four
-// chunks (about sixteen MFMAs) ahead, across slot boundaries, so their latency hides
+// which are mutually independent.  The global loads of the next tile are spread over
+// the step as well (dma(k) issues the k-th of NDMA instructions): issued back to back
+// after the barrier by all four waves they would hold every wave's issue slot, and
+// with one wave per SIMD the matrix pipe, for over a thousand cycles per step.
+// A scheduling fence after every chunk keeps the
+// compiler from regrouping them; the LDS operands of a chunk are requested three
+// chunks (about twelve MFMAs) ahead, across slot boundaries, so their latency hides
 // behind the chunks in between.
-template <typename Tr, int D>
+template <typename Tr, int D, int NDMA, typename Dma>
 __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
                                           const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16],
                                           f32x16 (&dkacc)[(D + 31) / 32], f32x16 (&dvacc)[(D + 31) / 32], float& csum,
-                                          float qk_scale, float colc, int lane) {
+                                          float qk_scale, float colc, int lane, Dma dma) {
   constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32, NCH = 8;
   constexpr int NC = (MB + 2) * NCH;  // chunks of the step: slots -1 .. MB
-  constexpr int PF = 4;               // LDS operands are requested this many chunks before their MFMAs
+  constexpr int PF = 3;               // LDS operands are requested this many chunks before their MFMAs
+  constexpr int kDmaEvery = (NC - NCH) / (NDMA > 0 ? NDMA : 1) > 0 ? (NC - NCH) / (NDMA > 0 ? NDMA : 1) : 1;
+  static_assert(NDMA * kDmaEvery <= NC - NCH, "every load instruction of the next tile finds a chunk");
   static_assert(KK <= NCH && 2 * DB <= NCH, "one k-step and one accumulation pair per chunk");
   const int g = lane >> 5, i = lane & 31;
   f32x16 s[MB], dp[MB];
@@ -145,6 +151,9 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
     constexpr int bs = slot + 1, bv = slot, bc = slot - 1;
     fetch(std::integral_constant<int, c + PF>{});
     if constexpr (u == NCH - PF) init_block(bs + 1);
+    // the next tile's load instructions, one every kDmaEvery chunks from the second slot on
+    if constexpr (c >= NCH && (c - NCH) % kDmaEvery == 0 && (c - NCH) / kDmaEvery < NDMA)
+      dma(std::integral_constant<int, (c - NCH) / kDmaEvery>{});
     if constexpr (do_s && u < KK) {
       s[bs] = Tr::mfma32(aq[c], kreg[u], s[bs]);
       dp[bs] = Tr::mfma32(ado[c], vreg[u], dp[bs]);
@@ -315,21 +324,42 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     if (n_diag == 0) issue(m_top, q_tile0, do_tile0);
     if (tid < BMQ) { rc_s0[tid] = rc_term(); dl_s0[tid] = dl_term(); }
   }
+  constexpr int PER = DirectTileLoader<D, BMQ>::PER;
   for (int t = 0; t < n_int; t += 2) {
     wait_vmem_all();
     __syncthreads();
-    if (t + 1 < n_int) issue(m_top - (t + 1) * BMQ, q_tile1, do_tile1);
-    dkdv_step_interior<Tr, D>(q_tile0, do_tile0, rc_s0, dl_s0, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane);
+    {  // tile t from buffers 0; tile t+1 (if any: otherwise an empty resource, the loads write zeros) into buffers 1
+      const bool more = t + 1 < n_int;
+      const int ms = m_top - (t + 1) * BMQ;
+      if (more) issue_rows(ms);
+      const uint16_t *q_next = qp + (int64_t)ms * a.q.st, *do_next = dop + (int64_t)ms * a.d_o.st;
+      const int q_bytes = qld.extent(a.q.st, ms, more ? M : ms), do_bytes = dold.extent(a.d_o.st, ms, more ? M : ms);
+      dkdv_step_interior<Tr, D, 2 * PER>(q_tile0, do_tile0, rc_s0, dl_s0, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane, [&](auto k) {
+        constexpr int K = decltype(k)::value;
+        if constexpr (K < PER) qld.issue_one(K, q_next, q_bytes, q_tile1);
+        else dold.issue_one(K - PER, do_next, do_bytes, do_tile1);
+      });
+    }
     if (t + 1 >= n_int) break;
     if (tid < BMQ) { rc_s1[tid] = rc_term(); dl_s1[tid] = dl_term(); }
     wait_vmem_all();
     __syncthreads();
-    if (t + 2 < n_int) issue(m_top - (t + 2) * BMQ, q_tile0, do_tile0);
-    dkdv_step_interior<Tr, D>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane);
-    if (t + 2 < n_int && tid < BMQ) { rc_s0[tid] = rc_term(); dl_s0[tid] = dl_term(); }
+    {
+      const bool more = t + 2 < n_int;
+      const int ms = m_top - (t + 2) * BMQ;
+      if (more) issue_rows(ms);
+      const uint16_t *q_next = qp + (int64_t)ms * a.q.st, *do_next = dop + (int64_t)ms * a.d_o.st;
+      const int q_bytes = qld.extent(a.q.st, ms, more ? M : ms), do_bytes = dold.extent(a.d_o.st, ms, more ? M : ms);
+      dkdv_step_interior<Tr, D, 2 * PER>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane, [&](auto k) {
+        constexpr int K = decltype(k)::value;
+        if constexpr (K < PER) qld.issue_one(K, q_next, q_bytes, q_tile0);
+        else dold.issue_one(K - PER, do_next, do_bytes, do_tile0);
+      });
+      if (more && tid < BMQ) { rc_s0[tid] = rc_term(); dl_s0[tid] = dl_term(); }
+    }
   }
 
-  if (early && n_steps == 0) wait_vmem_all();  // the requested tile must land before the workgroup's LDS is released
+  wait_vmem_all();  // whatever was requested last (possibly an empty tile) has landed before the buffers are reused
   const float ctot = half_sum(csum);
   if (n < N && g == 0) a.dc[(int64_t)bh * N + n] = -ctot;
   // dK and dV leave through LDS (the tile buffers are free now) so that the global stores are whole rows

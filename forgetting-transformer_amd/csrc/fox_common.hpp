@@ -205,16 +205,26 @@ struct DirectTileLoader {
       voff[j] = (int)(row * row_stride * 2) + (c << 4);
     }
   }
+  // Byte extent of the tile whose first row is row0, for its buffer resource: rows at or beyond row_limit
+  // are out of range, and an extent of 0 (row_limit <= row0) makes every load return zero.
+  __device__ __forceinline__ int extent(int64_t row_stride, int row0, int row_limit) const {
+    return row_limit > row0 ? (int)(((int64_t)(row_limit - 1 - row0) * row_stride + D) * 2) : 0;
+  }
+  // The j-th (a constant at every call site) of this wave's PER load instructions of the tile that
+  // starts at p, so that a kernel can spread them over its compute instead of issuing them back to back
+  // (each one occupies the wave's issue slot, and the CU's memory pipeline, for tens of cycles).
+  __device__ __forceinline__ void issue_one(int j, const uint16_t* p, int bytes, char* tile) const {
+    const int blk = wave + NW * j;
+    if (NBLK % NW == 0 || blk < NBLK) {
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, bytes, 0x00020000);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(tile + blk * Tile<D>::BLOCK_BYTES), 16, voff[j], 0, 0, 0);
+    }
+  }
   __device__ __forceinline__ void issue(const uint16_t* base, int64_t row_stride, int row0, int row_limit, char* tile) const {
     const uint16_t* p = base + (int64_t)row0 * row_stride;
-    const int64_t bytes = row_limit > row0 ? ((int64_t)(row_limit - 1 - row0) * row_stride + D) * 2 : 0;
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, (int)bytes, 0x00020000);
+    const int bytes = extent(row_stride, row0, row_limit);
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int blk = wave + NW * j;
-      if (NBLK % NW == 0 || blk < NBLK)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(tile + blk * Tile<D>::BLOCK_BYTES), 16, voff[j], 0, 0, 0);
-    }
+    for (int j = 0; j < PER; ++j) issue_one(j, p, bytes, tile);
   }
 };
 
