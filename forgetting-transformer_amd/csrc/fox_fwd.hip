@@ -111,11 +111,13 @@ __device__ __forceinline__ void fwd_tile(const char* k_tile, const char* v_tile,
 // accumulates the current tile's P V (from v_cur).  s_cur holds the raw scores of the current tile
 // on entry; s_next holds those of the next tile on exit.  Work is issued in small chunks separated
 // by scheduling fences so that MFMA and vector instructions alternate in the instruction stream.
-template <typename Tr, int D>
+// dma(u) issues chunk u's share of the global loads of the tiles after next: spread over the tile they
+// do not hold the wave's issue slot back to back right after the barrier.
+template <typename Tr, int D, typename Dma>
 __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const char* v_cur, const float* cn_next,
                                                   const u32x4 (&qreg)[D / 16], f32x16 (&oacc)[(D + 31) / 32], float& m_i,
                                                   float& l_i, float qk_scale, int lane, f32x16 (&s_cur)[kFwdBN / 32],
-                                                  f32x16 (&s_next)[kFwdBN / 32]) {
+                                                  f32x16 (&s_next)[kFwdBN / 32], Dma dma) {
   constexpr int BN = kFwdBN, KK = D / 16, DB = (D + 31) / 32, NB = BN / 32, NSL = BN / 16;
   constexpr int SPC = 16 * NB / KK;  // scores handled per chunk of phase A
   static_assert(16 * NB % KK == 0 && SPC % 4 == 0, "whole float4 groups of scores per chunk");
@@ -129,9 +131,10 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
     ka[nb][0] = lds_row_operand<D>(k_next, 32 * nb + i, g);
     s_next[nb] = acc_init(cn_next, 32 * nb, g);
   }
-#pragma unroll
-  for (int u = 0; u < KK; ++u) {
-    if (u + 1 < KK) {
+  static_for<0, KK>([&](auto uc) {
+    constexpr int u = decltype(uc)::value;
+    dma(u);  // this chunk's share of the global loads of the tiles after next
+    if constexpr (u + 1 < KK) {
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) ka[nb][u + 1] = lds_row_operand<D>(k_next, 32 * nb + i, 2 * (u + 1) + g);
     }
@@ -148,7 +151,7 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
       __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-  }
+  });
   mloc = half_max(mloc) * qk_scale;
   const bool raise = mloc > m_i + kLazyMaxLog2;
   if (__any(raise)) {  // rare: rescale what has been accumulated so far
@@ -199,6 +202,34 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
   }
   l_i += rsum;
 }
+
+// The global loads of a K tile and a V tile, dealt out over the D/16 chunks of a pipelined tile:
+// dma(u) issues chunk u's share.
+template <int D>
+struct TileDma {
+  static constexpr int KK = D / 16, PER = DirectTileLoader<D, kFwdBN>::PER, PER_CHUNK = (2 * PER + KK - 1) / KK;
+  const DirectTileLoader<D, kFwdBN>& kld;
+  const DirectTileLoader<D, kFwdBN>& vld;
+  const uint16_t* k_src;
+  const uint16_t* v_src;
+  int k_bytes, v_bytes;
+  char* k_fill;
+  char* v_fill;
+  __device__ __forceinline__ void all() const {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) kld.issue_one(j, k_src, k_bytes, k_fill);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) vld.issue_one(j, v_src, v_bytes, v_fill);
+  }
+  __device__ __forceinline__ void operator()(int u) const {  // u is a constant at every call site
+#pragma unroll
+    for (int r = 0; r < PER_CHUNK; ++r) {
+      const int idx = u * PER_CHUNK + r;
+      if (idx < PER) kld.issue_one(idx, k_src, k_bytes, k_fill);
+      else if (idx < 2 * PER) vld.issue_one(idx - PER, v_src, v_bytes, v_fill);
+    }
+  }
+};
 
 template <typename Tr, int D, bool SPLIT>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
@@ -360,23 +391,33 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) s_a[nb] = Tr::mfma32(lds_row_operand<D>(k_tile0, 32 * nb + i, 2 * kk + g), qreg[kk], s_a[nb]);
     }
+    // Iteration j: S(j+1) from k_nx, P(j) V(j) from v_cur; meanwhile K(j+2) is requested into k_fill and
+    // V(j+1) into v_fill, one load instruction per chunk of the tile (an empty extent when there is no such
+    // tile: the loads then write zeros into the free buffer).
+    auto pipelined_tile = [&](int j, const char* k_nx, const char* v_cur, const float* cn_nx, char* k_fill, char* v_fill,
+                              f32x16 (&s_cur)[NB], f32x16 (&s_nx)[NB]) {
+      const bool more_k = j + 2 < n_int, more_v = j + 1 < n_int;
+      const int nk = more_k ? lo + (n_int - 3 - j) * BN : lo, nv = more_v ? lo + (n_int - 2 - j) * BN : lo;
+      if (more_k) issue_cn(nk);
+      const uint16_t *k_src = kp + (int64_t)nk * a.k.st, *v_src = vp + (int64_t)nv * a.v.st;
+      const int k_bytes = kld.extent(a.k.st, nk, more_k ? N : nk), v_bytes = vld.extent(a.v.st, nv, more_v ? N : nv);
+      const TileDma<D> dma{kld, vld, k_src, v_src, k_bytes, v_bytes, k_fill, v_fill};
+      if (wave_has_rows) fwd_tile_pipelined<Tr, D>(k_nx, v_cur, cn_nx, qreg, oacc, m_i, l_i, qk_scale, lane, s_cur, s_nx, dma);
+      else dma.all();  // a wave without query rows only moves its share of the tiles
+    };
     for (int j = 0; j < n_int; j += 2) {
       // even iteration: K(j+1) in k_tile1 with its key terms in cn_s1, V(j) in v_tile0.  The key
       // terms of tile j+1 go to LDS before the barrier: their buffer was last read two iterations ago.
       wait_vmem_all();
       if (j + 1 < n_int && tid < BN) cn_s1[tid] = cn_term();
       __syncthreads();
-      if (j + 2 < n_int) issue_k(j + 2, k_tile0);
-      if (j + 1 < n_int) issue_v(j + 1, v_tile1);
-      if (wave_has_rows) fwd_tile_pipelined<Tr, D>(k_tile1, v_tile0, cn_s1, qreg, oacc, m_i, l_i, qk_scale, lane, s_a, s_b);
+      pipelined_tile(j, k_tile1, v_tile0, cn_s1, k_tile0, v_tile1, s_a, s_b);
       if (j + 1 >= n_int) break;
       // odd iteration: K(j+2) in k_tile0 with its key terms in cn_s0, V(j+1) in v_tile1
       wait_vmem_all();
       if (j + 2 < n_int && tid < BN) cn_s0[tid] = cn_term();
       __syncthreads();
-      if (j + 3 < n_int) issue_k(j + 3, k_tile1);
-      if (j + 2 < n_int) issue_v(j + 2, v_tile0);
-      if (wave_has_rows) fwd_tile_pipelined<Tr, D>(k_tile0, v_tile1, cn_s0, qreg, oacc, m_i, l_i, qk_scale, lane, s_b, s_a);
+      pipelined_tile(j + 1, k_tile0, v_tile1, cn_s0, k_tile1, v_tile0, s_b, s_a);
     }
   }
 
@@ -410,6 +451,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   if (m < M && g == 0) a.lse[(int64_t)bh * M + m] = empty ? -INFINITY : (m_i + cm2) * kLn2 + __logf(l_tot);
   // o leaves through LDS (the tile buffers are free now, one per wave) so that the global stores are whole rows
   static_assert(kStoreStageBytes<D> <= Tile<D>::bytes(BN), "one wave stages in one tile buffer");
+  wait_vmem_all();  // whatever was requested last (possibly an empty tile) has landed
   __syncthreads();  // every wave is done with the last tile
   char* stage = wave == 0 ? k_tile0 : wave == 1 ? k_tile1 : wave == 2 ? v_tile0 : v_tile1;
   store_rows_via_lds<Tr, D>(stage, oacc, inv, op, a.o.st, m0 + 32 * wave, M, lane);
