@@ -258,11 +258,15 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   // Per-row terms of a step: the loads are requested here, the arithmetic on them is done where the values
   // go to LDS (a step later), so that nothing waits for the loads in between.  Rows past M and empty rows
   // (lse = -inf) get -inf through the subtraction.
+  // The BMQ rows of a step are dealt out evenly over the four waves (their first BMQ/4 lanes each), so that
+  // no wave arrives late at the barrier because of them.
+  const bool row_lane = lane < BMQ / 4;
+  const int row_slot = wave * (BMQ / 4) + lane;
   float l_raw = 0.f, c_raw = 0.f, d_raw = 0.f;
   bool row_ok = false;
   auto issue_rows = [&](int ms) {
-    if (tid < BMQ) {
-      const int mm = ms + tid, mc = min(mm, M - 1);
+    if (row_lane) {
+      const int mm = ms + row_slot, mc = min(mm, M - 1);
       row_ok = mm < M;
       l_raw = lse_row[mc];
       c_raw = c_row[p_seq + mc];
@@ -314,7 +318,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
       __syncthreads();  // buffer 1 is free again
       issue(ms, q_tile1, do_tile1);
     }
-    if (tid < BMQ) { rc_s1[tid] = rc_term(); dl_s1[tid] = dl_term(); }
+    if (row_lane) { rc_s1[row_slot] = rc_term(); dl_s1[row_slot] = dl_term(); }
     wait_vmem_all();
     __syncthreads();
     if (t == n_diag - 1 && n_int > 0) issue(m_top, q_tile0, do_tile0);
@@ -322,7 +326,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
   }
   if (n_int > 0) {
     if (n_diag == 0) issue(m_top, q_tile0, do_tile0);
-    if (tid < BMQ) { rc_s0[tid] = rc_term(); dl_s0[tid] = dl_term(); }
+    if (row_lane) { rc_s0[row_slot] = rc_term(); dl_s0[row_slot] = dl_term(); }
   }
   constexpr int PER = DirectTileLoader<D, BMQ>::PER;
   for (int t = 0; t < n_int; t += 2) {
@@ -341,7 +345,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
       });
     }
     if (t + 1 >= n_int) break;
-    if (tid < BMQ) { rc_s1[tid] = rc_term(); dl_s1[tid] = dl_term(); }
+    if (row_lane) { rc_s1[row_slot] = rc_term(); dl_s1[row_slot] = dl_term(); }
     wait_vmem_all();
     __syncthreads();
     {
@@ -355,7 +359,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
         if constexpr (K < PER) qld.issue_one(K, q_next, q_bytes, q_tile0);
         else dold.issue_one(K - PER, do_next, do_bytes, do_tile0);
       });
-      if (more && tid < BMQ) { rc_s0[tid] = rc_term(); dl_s0[tid] = dl_term(); }
+      if (more && row_lane) { rc_s0[row_slot] = rc_term(); dl_s0[row_slot] = dl_term(); }
     }
   }
 
