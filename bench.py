@@ -363,6 +363,13 @@ def norm_gate_report(ns):
     bytes_f, bytes_b = 3 * S + rows * G * 4, 5 * S + rows * G * 4 + 2 * nb.value
     kernels = {"norm_gate_fwd": {"ms": t_f * 1e3, "gbps": bytes_f / t_f * 1e-9, "algorithmic_bytes": bytes_f},
                "norm_gate_bwd": {"ms": t_b * 1e3, "gbps": bytes_b / t_b * 1e-9, "algorithmic_bytes": bytes_b}}
+    # the same kernels without a gate: the per-head RMS norm of queries and keys (QK-norm); one tensor less each way
+    args.activation, args.g, args.dg = _lib.ACT_NONE, None, None
+    t_pf = event_time(lambda: _lib.check(lib.fox_norm_gate_fwd(C.byref(args), stream), "norm fwd"), max(5, ns.steps))
+    t_pb = event_time(lambda: _lib.check(lib.fox_norm_gate_bwd(C.byref(args), stream), "norm bwd"), max(5, ns.steps))
+    bytes_pf, bytes_pb = 2 * S + rows * G * 4, 3 * S + rows * G * 4 + 2 * nb.value
+    kernels["qk_norm_fwd"] = {"ms": t_pf * 1e3, "gbps": bytes_pf / t_pf * 1e-9, "algorithmic_bytes": bytes_pf}
+    kernels["qk_norm_bwd"] = {"ms": t_pb * 1e3, "gbps": bytes_pb / t_pb * 1e-9, "algorithmic_bytes": bytes_pb}
     line = {
         "metric": "gated per-head RMS norm fwd+bwd, algorithmic HBM GB/s (operator incl. autograd)",
         "value": (bytes_f + bytes_b) / sec * 1e-9, "unit": "GB/s", "n_gpus": 1, "steps": ns.steps, "warmup": ns.warmup,

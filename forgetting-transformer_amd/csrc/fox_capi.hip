@@ -127,22 +127,27 @@ int make_norm_gate(const fox_norm_gate_args* a, fox::NormGateK& k, bool bwd) {
   if (a->rows <= 0 || a->G <= 0) return fail(FOX_E_ARG, "rows and G must be positive");
   if (a->D != 16 && a->D != 32 && a->D != 64 && a->D != 128) return fail(FOX_E_ARG, "head dim must be one of 16, 32, 64, 128 (got %d)", a->D);
   if (a->dtype != FOX_DTYPE_BF16 && a->dtype != FOX_DTYPE_FP16) return fail(FOX_E_ARG, "dtype must be FOX_DTYPE_BF16 or FOX_DTYPE_FP16 (got %d)", a->dtype);
-  if (a->activation != FOX_ACT_SIGMOID && a->activation != FOX_ACT_SWISH) return fail(FOX_E_ARG, "activation must be FOX_ACT_SIGMOID or FOX_ACT_SWISH (got %d)", a->activation);
+  if (a->activation != FOX_ACT_SIGMOID && a->activation != FOX_ACT_SWISH && a->activation != FOX_ACT_NONE) return fail(FOX_E_ARG, "activation must be FOX_ACT_SIGMOID, FOX_ACT_SWISH or FOX_ACT_NONE (got %d)", a->activation);
+  const bool gated = a->activation != FOX_ACT_NONE;
   if (a->rows * a->G * (a->D / 8) > ((int64_t)1 << 39)) return fail(FOX_E_ARG, "tensor too large");
-  if (!a->x || !a->g || !a->weight || !a->rstd) return fail(FOX_E_ARG, "x, g, weight and rstd must not be NULL");
-  const void* ptrs[6] = {a->x, a->g, bwd ? a->dy : a->y, bwd ? a->dx : a->y, bwd ? a->dg : a->y, a->weight};
-  const int64_t strides[6] = {a->x_stride_row, a->g_stride_row, bwd ? a->dy_stride_row : a->y_stride_row,
-                              bwd ? a->dx_stride_row : a->y_stride_row, bwd ? a->dg_stride_row : a->y_stride_row, 8};
+  if (!a->x || !a->weight || !a->rstd) return fail(FOX_E_ARG, "x, weight and rstd must not be NULL");
+  if (gated && !a->g) return fail(FOX_E_ARG, "g must not be NULL for a gated activation");
+  // the ungated form neither reads g nor writes dg: both are ignored and may be NULL
+  const void* ptrs[6] = {a->x, gated ? a->g : a->x, bwd ? a->dy : a->y, bwd ? a->dx : a->y,
+                         bwd ? (gated ? a->dg : a->dx) : a->y, a->weight};
+  const int64_t strides[6] = {a->x_stride_row, gated ? a->g_stride_row : 8, bwd ? a->dy_stride_row : a->y_stride_row,
+                              bwd ? a->dx_stride_row : a->y_stride_row,
+                              bwd ? (gated ? a->dg_stride_row : 8) : a->y_stride_row, 8};
   for (int i = 0; i < 6; ++i) {
-    if (!ptrs[i]) return fail(FOX_E_ARG, bwd ? "dy, dx and dg must not be NULL" : "y must not be NULL");
+    if (!ptrs[i]) return fail(FOX_E_ARG, bwd ? "dy, dx and (for a gated activation) dg must not be NULL" : "y must not be NULL");
     if (((uintptr_t)ptrs[i] & 15) != 0) return fail(FOX_E_ALIGN, "tensors must be 16-byte aligned");
     if (strides[i] & 7) return fail(FOX_E_ALIGN, "row strides must be multiples of 8 elements");
   }
   if (bwd && (!a->dweight || !a->workspace)) return fail(FOX_E_ARG, "dweight and workspace must not be NULL");
   if (bwd && ((uintptr_t)a->workspace & 15) != 0) return fail(FOX_E_ALIGN, "workspace must be 16-byte aligned");
   k = fox::NormGateK{};
-  k.x = (const uint16_t*)a->x; k.g = (const uint16_t*)a->g; k.y = (uint16_t*)a->y;
-  k.dy = (const uint16_t*)a->dy; k.dx = (uint16_t*)a->dx; k.dg = (uint16_t*)a->dg;
+  k.x = (const uint16_t*)a->x; k.g = gated ? (const uint16_t*)a->g : nullptr; k.y = (uint16_t*)a->y;
+  k.dy = (const uint16_t*)a->dy; k.dx = (uint16_t*)a->dx; k.dg = gated ? (uint16_t*)a->dg : nullptr;
   k.w = a->weight; k.rstd = a->rstd; k.dw = a->dweight; k.dw_partial = a->workspace;
   k.x_sr = a->x_stride_row; k.g_sr = a->g_stride_row; k.y_sr = a->y_stride_row;
   k.dy_sr = a->dy_stride_row; k.dx_sr = a->dx_stride_row; k.dg_sr = a->dg_stride_row;
@@ -170,14 +175,14 @@ int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_b
 int fox_norm_gate_fwd(const fox_norm_gate_args* args, void* stream) {
   fox::NormGateK k;
   FOX_TRY(make_norm_gate(args, k, false));
-  return check_hip(fox::launch_norm_gate(k, args->D, args->dtype, false, args->activation == FOX_ACT_SWISH, (hipStream_t)stream),
+  return check_hip(fox::launch_norm_gate(k, args->D, args->dtype, false, args->activation, (hipStream_t)stream),
                    "fox_norm_gate_fwd");
 }
 
 int fox_norm_gate_bwd(const fox_norm_gate_args* args, void* stream) {
   fox::NormGateK k;
   FOX_TRY(make_norm_gate(args, k, true));
-  return check_hip(fox::launch_norm_gate(k, args->D, args->dtype, true, args->activation == FOX_ACT_SWISH, (hipStream_t)stream),
+  return check_hip(fox::launch_norm_gate(k, args->D, args->dtype, true, args->activation, (hipStream_t)stream),
                    "fox_norm_gate_bwd");
 }
 

@@ -1,12 +1,15 @@
-// Gated per-head RMS normalisation for gfx950: the epilogue the FoX layer applies to the
-// attention output before the output projection,
+// Per-head RMS normalisation for gfx950, gated or plain: the epilogue the FoX layer applies to the
+// attention output before the output projection, and the normalisation of queries and keys in front
+// of the attention (QK-norm),
 //   y[r,h,:] = x[r,h,:] * rstd[r,h] * w[h,:] * act(g[r,h,:]),   rstd = 1 / sqrt(mean_d x^2 + eps),
-// act(g) = sigmoid(g) or g*sigmoid(g) (swish), and its backward
+// act(g) = sigmoid(g), g*sigmoid(g) (swish) or 1 (no gate tensor), and its backward
 //   yn = xhat * w (xhat = x * rstd),  dg = dy * yn * act'(g),  dyn = dy * act(g),
 //   dw[h,:] = sum_r dyn * xhat,  dx = (dyn*w - xhat * mean_d(dyn*w*xhat)) * rstd.
 // (reference: model/forgetting_transformer/fuse_norm_gate.py:132-206 forward, :309-417 backward, the
 // configuration FusedGroupNormGated(num_groups=heads, is_rms_norm=True, activation="sigmoid") of
-// modeling_forgetting_transformer.py:243, no bias, no residual)
+// modeling_forgetting_transformer.py:243, no bias, no residual; the plain form is layer_norm_fwd_kernel /
+// layer_norm_bwd_kernel of layernorm.py:183-254, :328-435 as used by GroupNorm(num_groups=heads,
+// is_rms_norm=True) and RMSNorm(head_dim), modeling_forgetting_transformer.py:258-265, :314-325)
 //
 // Both are pure streams over HBM.  A (row, head) group of D elements is spread over D/8 lanes, 16
 // bytes each; the two row reductions are shuffles inside that lane group.  In the backward every
@@ -35,7 +38,9 @@ __device__ __forceinline__ u32x4 pack8v(const float (&f)[8]) {
 }
 __device__ __forceinline__ float sigmoidf(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
-template <typename Tr, int D, bool SWISH>
+enum : int { kActSigmoid = 0, kActSwish = 1, kActNone = 2 };  // FOX_ACT_* of the public header
+
+template <typename Tr, int D, int ACT>
 __global__ __launch_bounds__(256) void norm_gate_fwd_kernel(const NormGateK a) {
   constexpr int CH = D / 8;
   const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -47,7 +52,7 @@ __global__ __launch_bounds__(256) void norm_gate_fwd_kernel(const NormGateK a) {
   const int64_t off = h * (int64_t)D + chunk * 8;
   float x[8], g[8], w[8], y[8];
   unpack8v<Tr>(*reinterpret_cast<const u32x4*>(a.x + row * a.x_sr + off), x);
-  unpack8v<Tr>(*reinterpret_cast<const u32x4*>(a.g + row * a.g_sr + off), g);
+  if (ACT != kActNone) unpack8v<Tr>(*reinterpret_cast<const u32x4*>(a.g + row * a.g_sr + off), g);
   {
     const f32x4 w0 = *reinterpret_cast<const f32x4*>(a.w + off), w1 = *reinterpret_cast<const f32x4*>(a.w + off + 4);
 #pragma unroll
@@ -61,8 +66,11 @@ __global__ __launch_bounds__(256) void norm_gate_fwd_kernel(const NormGateK a) {
   const float rstd = 1.0f / sqrtf(ss / D + a.eps);
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const float s = sigmoidf(g[e]);
-    y[e] = x[e] * rstd * w[e] * (SWISH ? g[e] * s : s);
+    y[e] = x[e] * rstd * w[e];
+    if (ACT != kActNone) {
+      const float s = sigmoidf(g[e]);
+      y[e] *= ACT == kActSwish ? g[e] * s : s;
+    }
   }
   if (live) {
     *reinterpret_cast<u32x4*>(a.y + row * a.y_sr + off) = pack8v<Tr>(y);
@@ -72,7 +80,7 @@ __global__ __launch_bounds__(256) void norm_gate_fwd_kernel(const NormGateK a) {
 
 constexpr int kNormStrip = 32;  // rows per thread in the backward
 
-template <typename Tr, int D, bool SWISH>
+template <typename Tr, int D, int ACT>
 __global__ __launch_bounds__(256) void norm_gate_bwd_kernel(const NormGateK a) {
   constexpr int CH = D / 8;
   const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -102,7 +110,7 @@ __global__ __launch_bounds__(256) void norm_gate_bwd_kernel(const NormGateK a) {
     for (int u = 0; u < U; ++u) {
       const int64_t r = min(rb + u, r1 - 1);
       xv[u] = *reinterpret_cast<const u32x4*>(a.x + r * a.x_sr + off);
-      gv[u] = *reinterpret_cast<const u32x4*>(a.g + r * a.g_sr + off);
+      if (ACT != kActNone) gv[u] = *reinterpret_cast<const u32x4*>(a.g + r * a.g_sr + off);
       dyv[u] = *reinterpret_cast<const u32x4*>(a.dy + r * a.dy_sr + off);
       rs[u] = a.rstd[r * a.G + hh];
     }
@@ -112,21 +120,23 @@ __global__ __launch_bounds__(256) void norm_gate_bwd_kernel(const NormGateK a) {
       if (r < r1) {  // uniform over the lanes of a (head, strip) group
         float x[8], g[8], dy[8], dx[8], dg[8], wdy[8];
         unpack8v<Tr>(xv[u], x);
-        unpack8v<Tr>(gv[u], g);
+        if (ACT != kActNone) unpack8v<Tr>(gv[u], g);
         unpack8v<Tr>(dyv[u], dy);
         float c1 = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float xhat = x[e] * rs[u];
           const float yn = xhat * w[e];
-          const float s = sigmoidf(g[e]);
-          float dyn;
-          if (SWISH) {
-            dg[e] = dy[e] * yn * (s + g[e] * s * (1.f - s));
-            dyn = dy[e] * g[e] * s;
-          } else {
-            dg[e] = dy[e] * yn * s * (1.f - s);
-            dyn = dy[e] * s;
+          float dyn = dy[e];
+          if (ACT != kActNone) {
+            const float s = sigmoidf(g[e]);
+            if (ACT == kActSwish) {
+              dg[e] = dy[e] * yn * (s + g[e] * s * (1.f - s));
+              dyn = dy[e] * g[e] * s;
+            } else {
+              dg[e] = dy[e] * yn * s * (1.f - s);
+              dyn = dy[e] * s;
+            }
           }
           dw[e] += dyn * xhat;
           wdy[e] = dyn * w[e];
@@ -139,7 +149,7 @@ __global__ __launch_bounds__(256) void norm_gate_bwd_kernel(const NormGateK a) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) dx[e] = (wdy[e] - x[e] * c1) * rs[u];
         *reinterpret_cast<u32x4*>(a.dx + r * a.dx_sr + off) = pack8v<Tr>(dx);
-        *reinterpret_cast<u32x4*>(a.dg + r * a.dg_sr + off) = pack8v<Tr>(dg);
+        if (ACT != kActNone) *reinterpret_cast<u32x4*>(a.dg + r * a.dg_sr + off) = pack8v<Tr>(dg);
       }
     }
   }
@@ -175,10 +185,12 @@ __global__ __launch_bounds__(256) void reduce_rows_kernel(const float* __restric
 }
 
 #define FOX_NG_INST(TR, DD)                                                   \
-  template __global__ void norm_gate_fwd_kernel<TR, DD, false>(const NormGateK); \
-  template __global__ void norm_gate_fwd_kernel<TR, DD, true>(const NormGateK);  \
-  template __global__ void norm_gate_bwd_kernel<TR, DD, false>(const NormGateK); \
-  template __global__ void norm_gate_bwd_kernel<TR, DD, true>(const NormGateK);
+  template __global__ void norm_gate_fwd_kernel<TR, DD, kActSigmoid>(const NormGateK); \
+  template __global__ void norm_gate_fwd_kernel<TR, DD, kActSwish>(const NormGateK);   \
+  template __global__ void norm_gate_fwd_kernel<TR, DD, kActNone>(const NormGateK);    \
+  template __global__ void norm_gate_bwd_kernel<TR, DD, kActSigmoid>(const NormGateK); \
+  template __global__ void norm_gate_bwd_kernel<TR, DD, kActSwish>(const NormGateK);   \
+  template __global__ void norm_gate_bwd_kernel<TR, DD, kActNone>(const NormGateK);
 #define FOX_NG_INST_ALL(TR) FOX_NG_INST(TR, 16) FOX_NG_INST(TR, 32) FOX_NG_INST(TR, 64) FOX_NG_INST(TR, 128)
 FOX_NG_INST_ALL(Bf16)
 FOX_NG_INST_ALL(Fp16)
@@ -191,20 +203,22 @@ int64_t norm_gate_workspace_rows(int64_t rows) {
 }
 
 template <typename Tr, int D>
-static hipError_t norm_gate_d(const NormGateK& a, bool bwd, bool swish, hipStream_t s) {
+static hipError_t norm_gate_d(const NormGateK& a, bool bwd, int act, hipStream_t s) {
   constexpr int CH = D / 8;
   if (!bwd) {
     const int64_t threads = (int64_t)a.R * a.G * CH;
     const dim3 grid((unsigned)((threads + 255) / 256));
-    if (swish) hipLaunchKernelGGL((norm_gate_fwd_kernel<Tr, D, true>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((norm_gate_fwd_kernel<Tr, D, false>), grid, dim3(256), 0, s, a);
+    if (act == kActSwish) hipLaunchKernelGGL((norm_gate_fwd_kernel<Tr, D, kActSwish>), grid, dim3(256), 0, s, a);
+    else if (act == kActNone) hipLaunchKernelGGL((norm_gate_fwd_kernel<Tr, D, kActNone>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((norm_gate_fwd_kernel<Tr, D, kActSigmoid>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
   }
   const int64_t strips = norm_gate_strips(a.R);
   const int64_t threads = strips * a.G * CH;
   const dim3 grid((unsigned)((threads + 255) / 256));
-  if (swish) hipLaunchKernelGGL((norm_gate_bwd_kernel<Tr, D, true>), grid, dim3(256), 0, s, a);
-  else hipLaunchKernelGGL((norm_gate_bwd_kernel<Tr, D, false>), grid, dim3(256), 0, s, a);
+  if (act == kActSwish) hipLaunchKernelGGL((norm_gate_bwd_kernel<Tr, D, kActSwish>), grid, dim3(256), 0, s, a);
+  else if (act == kActNone) hipLaunchKernelGGL((norm_gate_bwd_kernel<Tr, D, kActNone>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((norm_gate_bwd_kernel<Tr, D, kActSigmoid>), grid, dim3(256), 0, s, a);
   const int width = a.G * D;
   const int64_t groups = (strips + kReduceGroup - 1) / kReduceGroup;
   float* stage = a.dw_partial + strips * width;  // second part of the workspace
@@ -216,18 +230,18 @@ static hipError_t norm_gate_d(const NormGateK& a, bool bwd, bool swish, hipStrea
 }
 
 template <typename Tr>
-static hipError_t norm_gate_t(const NormGateK& a, int D, bool bwd, bool swish, hipStream_t s) {
+static hipError_t norm_gate_t(const NormGateK& a, int D, bool bwd, int act, hipStream_t s) {
   switch (D) {
-    case 16: return norm_gate_d<Tr, 16>(a, bwd, swish, s);
-    case 32: return norm_gate_d<Tr, 32>(a, bwd, swish, s);
-    case 64: return norm_gate_d<Tr, 64>(a, bwd, swish, s);
-    case 128: return norm_gate_d<Tr, 128>(a, bwd, swish, s);
+    case 16: return norm_gate_d<Tr, 16>(a, bwd, act, s);
+    case 32: return norm_gate_d<Tr, 32>(a, bwd, act, s);
+    case 64: return norm_gate_d<Tr, 64>(a, bwd, act, s);
+    case 128: return norm_gate_d<Tr, 128>(a, bwd, act, s);
     default: return hipErrorInvalidValue;
   }
 }
 
-hipError_t launch_norm_gate(const NormGateK& a, int D, int dtype, bool bwd, bool swish, hipStream_t s) {
-  return dtype == 0 ? norm_gate_t<Bf16>(a, D, bwd, swish, s) : norm_gate_t<Fp16>(a, D, bwd, swish, s);
+hipError_t launch_norm_gate(const NormGateK& a, int D, int dtype, bool bwd, int act, hipStream_t s) {
+  return dtype == 0 ? norm_gate_t<Bf16>(a, D, bwd, act, s) : norm_gate_t<Fp16>(a, D, bwd, act, s);
 }
 
 }  // namespace fox

@@ -1,5 +1,6 @@
-from .forgetting_attention import forgetting_attention, forgetting_attention_from_logits
-from .norm_gate import group_norm_gated
+from .forgetting_attention import forgetting_attention, forgetting_attention_from_logits, qk_norm_threshold
+from .norm_gate import group_norm, group_norm_gated, rms_norm
 from .token_shift import token_shift
 
-__all__ = ["forgetting_attention", "forgetting_attention_from_logits", "group_norm_gated", "token_shift"]
+__all__ = ["forgetting_attention", "forgetting_attention_from_logits", "qk_norm_threshold", "group_norm",
+           "group_norm_gated", "rms_norm", "token_shift"]

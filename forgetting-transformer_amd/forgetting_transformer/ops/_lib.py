@@ -75,6 +75,7 @@ class ShiftArgs(C.Structure):
 
 ACT_SIGMOID = 0
 ACT_SWISH = 1
+ACT_NONE = 2
 
 
 class NormGateArgs(C.Structure):

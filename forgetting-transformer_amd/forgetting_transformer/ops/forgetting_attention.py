@@ -20,7 +20,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["forgetting_attention", "forgetting_attention_from_logits", "ForgettingAttention",
+__all__ = ["forgetting_attention", "forgetting_attention_from_logits", "qk_norm_threshold", "ForgettingAttention",
            "ForgettingAttentionFromLogits"]
 
 _DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
@@ -326,3 +326,25 @@ def forgetting_attention_from_logits(
     if not head_first:
         out, log_fgate = out.transpose(1, 2), log_fgate.transpose(1, 2)
     return out, log_fgate
+
+
+@torch.no_grad()
+def qk_norm_threshold(q_norm_weight: torch.Tensor, k_norm_weight: torch.Tensor, num_heads: int, head_dim: int,
+                      seq_len: int, log_pruning_tolerance: float, share_param_across_head: bool = False) -> torch.Tensor:
+    """``adaptive_threshold`` for queries and keys that went through an RMS QK-norm, from the norm weights alone.
+
+    The caller-side rule of the FoX layer (``modeling_forgetting_transformer.py:366-380``): a normalised row has
+    L2 norm at most ``max|w| * sqrt(head_dim)``, so with ``sm_scale = 1/sqrt(head_dim)`` no logit exceeds
+    ``max|w_q| * max|w_k| * sqrt(head_dim)``; the threshold is ``-(2 * bound + log(seq_len)) + log_pruning_tolerance``.
+    Weights of shape ``(num_heads * head_dim,)`` give one threshold per head, shape ``(num_heads,)``, which
+    ``forgetting_attention`` broadcasts over the batch; with ``share_param_across_head`` the weights are
+    ``(head_dim,)`` and the result is a 0-d tensor.  No pass over q and k is needed (unlike ``"auto"``).
+    """
+    if share_param_across_head:
+        assert q_norm_weight.shape == k_norm_weight.shape == (head_dim,)
+        bound = q_norm_weight.abs().max() * k_norm_weight.abs().max() * math.sqrt(head_dim)
+    else:
+        assert q_norm_weight.shape == k_norm_weight.shape == (num_heads * head_dim,)
+        bound = (q_norm_weight.view(num_heads, head_dim).abs().max(dim=-1).values
+                 * k_norm_weight.view(num_heads, head_dim).abs().max(dim=-1).values * math.sqrt(head_dim))
+    return -(2 * bound + math.log(seq_len)) + log_pruning_tolerance

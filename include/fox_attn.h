@@ -193,17 +193,21 @@ int fox_token_shift_fwd(const fox_shift_args* args, void* stream);
 int fox_token_shift_bwd(const fox_shift_args* args, void* stream);
 
 /*
- * Gated per-head RMS normalisation, the epilogue the FoX layer applies to the attention output before the
- * output projection (FusedGroupNormGated(num_groups=heads, is_rms_norm=True, activation="sigmoid"),
- * model/forgetting_transformer/modeling_forgetting_transformer.py:243, :417-420):
+ * Per-head RMS normalisation, gated or plain.  Gated: the epilogue the FoX layer applies to the attention
+ * output before the output projection (FusedGroupNormGated(num_groups=heads, is_rms_norm=True,
+ * activation="sigmoid"), model/forgetting_transformer/modeling_forgetting_transformer.py:243, :417-420).
+ * Plain (FOX_ACT_NONE; g and dg are ignored and may be NULL): the normalisation of queries and keys in
+ * front of the attention, GroupNorm(num_groups=heads, is_rms_norm=True) or RMSNorm(head_dim) (:258-265,
+ * :314-325; the latter is G = 1 with one row per (token, head)), and the ungated output norm (:245).
  *   y[r,h,:] = x[r,h,:] * rstd[r,h] * weight[h,:] * act(g[r,h,:]),  rstd = 1/sqrt(mean_d x[r,h,:]^2 + eps),
- * act = sigmoid (FOX_ACT_SIGMOID) or g*sigmoid(g) (FOX_ACT_SWISH).  x, g, y, dy, dx, dg are 16-bit tensors of
+ * act = sigmoid (FOX_ACT_SIGMOID), g*sigmoid(g) (FOX_ACT_SWISH) or 1 (FOX_ACT_NONE).  x, g, y, dy, dx, dg are 16-bit tensors of
  * `rows` rows of G*D contiguous elements, each with its own row stride in elements (a multiple of 8, base
  * pointers 16-byte aligned); weight and dweight are G*D fp32; rstd is (rows, G) fp32, written by the
  * forward and read by the backward.  No bias, no residual.  D is one of 16, 32, 64, 128.
  */
 #define FOX_ACT_SIGMOID 0
 #define FOX_ACT_SWISH 1
+#define FOX_ACT_NONE 2
 
 typedef struct fox_norm_gate_args {
   int64_t rows;
@@ -223,12 +227,14 @@ typedef struct fox_norm_gate_args {
   float* workspace;     /* fox_norm_gate_workspace_bytes() bytes, 16-byte aligned */
 } fox_norm_gate_args;
 
-/* Replaces layer_norm_gated_fwd_kernel as launched by LayerNormGatedFunction.forward (fuse_norm_gate.py:132-206, :539-618). */
+/* Replaces layer_norm_gated_fwd_kernel as launched by LayerNormGatedFunction.forward (fuse_norm_gate.py:132-206, :539-618)
+ * and, with FOX_ACT_NONE, layer_norm_fwd_kernel as launched by LayerNormFunction.forward (layernorm.py:183-254, :520-600). */
 int fox_norm_gate_fwd(const fox_norm_gate_args* args, void* stream);
 
 /*
  * dx, dg and dweight = sum over rows of dy*act(g)*xhat.  Replaces layer_norm_gated_bwd_kernel and the sum over
- * its partial weight gradients (fuse_norm_gate.py:309-417, :620-724).  The partial sums live in `workspace`
+ * its partial weight gradients (fuse_norm_gate.py:309-417, :620-724; with FOX_ACT_NONE layer_norm_bwd_kernel,
+ * layernorm.py:328-435, :603-703; dg is then not written).  The partial sums live in `workspace`
  * and are added in a fixed order, so the result is reproducible bit for bit.
  */
 int fox_norm_gate_bwd(const fox_norm_gate_args* args, void* stream);

@@ -24,7 +24,8 @@
  *                                           dprev = <dout[t], x[t-1]>
  *
  * and (src/forgetting_transformer/model/forgetting_transformer/fuse_norm_gate.py):
- *   fox_oracle_norm_gate_fwd/bwd :132-206, :309-417  per-group RMS norm * weight * sigmoid(g) (swish = 1: g*sigmoid(g)),
+ *   fox_oracle_norm_gate_fwd/bwd :132-206, :309-417  per-group RMS norm * weight * sigmoid(g) (swish = 1: g*sigmoid(g);
+ *                                                     swish = 2: no gate, g and dg untouched = layernorm.py:183-254, :328-435),
  *                                           dx, dg, dweight as in the backward kernel
  *
  * Layouts: q,out,dout,dq are (B,H,M,D); k,v,dk,dv are (B,H,N,D); c,dc,dg are (B,H,N);
@@ -230,7 +231,18 @@ void fox_oracle_token_shift_bwd(const double* x, const double* prev_w, const dou
 }
 
 
-/* Gated per-group RMS norm: x, g, y, dy, dx, dg are (R, G, D) contiguous doubles; w, dw are (G, D). */
+/* Gated per-group RMS norm: x, g, y, dy, dx, dg are (R, G, D) contiguous doubles; w, dw are (G, D).
+ * swish: 0 = sigmoid gate, 1 = swish gate, 2 = no gate (g is not read, dg is not written). */
+static double gate_act(const double* g, int64_t i, int mode) {
+  if (mode == 2) return 1.0;
+  const double s = 1.0 / (1.0 + exp(-g[i]));
+  return mode ? g[i] * s : s;
+}
+static double gate_dact(const double* g, int64_t i, int mode) {
+  if (mode == 2) return 0.0;
+  const double s = 1.0 / (1.0 + exp(-g[i]));
+  return mode ? s + g[i] * s * (1.0 - s) : s * (1.0 - s);
+}
 void fox_oracle_norm_gate_fwd(const double* x, const double* g, const double* w, double* y, int64_t R, int G, int D, double eps,
                               int swish) {
   for (int64_t r = 0; r < R; ++r)
@@ -239,10 +251,7 @@ void fox_oracle_norm_gate_fwd(const double* x, const double* g, const double* w,
       double ss = 0.0;
       for (int d = 0; d < D; ++d) ss += x[o + d] * x[o + d];
       const double rstd = 1.0 / sqrt(ss / D + eps);
-      for (int d = 0; d < D; ++d) {
-        const double s = 1.0 / (1.0 + exp(-g[o + d]));
-        y[o + d] = x[o + d] * rstd * w[h * D + d] * (swish ? g[o + d] * s : s);
-      }
+      for (int d = 0; d < D; ++d) y[o + d] = x[o + d] * rstd * w[h * D + d] * gate_act(g, o + d, swish);
     }
 }
 
@@ -257,19 +266,16 @@ void fox_oracle_norm_gate_bwd(const double* x, const double* g, const double* w,
       const double rstd = 1.0 / sqrt(ss / D + eps);
       double c1 = 0.0;
       for (int d = 0; d < D; ++d) {
-        const double xhat = x[o + d] * rstd, s = 1.0 / (1.0 + exp(-g[o + d]));
-        const double act = swish ? g[o + d] * s : s;
-        const double dact = swish ? s + g[o + d] * s * (1.0 - s) : s * (1.0 - s);
-        dg[o + d] = dy[o + d] * xhat * w[h * D + d] * dact;
-        const double dyn = dy[o + d] * act;
+        const double xhat = x[o + d] * rstd;
+        if (swish != 2) dg[o + d] = dy[o + d] * xhat * w[h * D + d] * gate_dact(g, o + d, swish);
+        const double dyn = dy[o + d] * gate_act(g, o + d, swish);
         dw[h * D + d] += dyn * xhat;
         c1 += xhat * dyn * w[h * D + d];
       }
       c1 /= D;
       for (int d = 0; d < D; ++d) {
-        const double xhat = x[o + d] * rstd, s = 1.0 / (1.0 + exp(-g[o + d]));
-        const double act = swish ? g[o + d] * s : s;
-        dx[o + d] = (dy[o + d] * act * w[h * D + d] - xhat * c1) * rstd;
+        const double xhat = x[o + d] * rstd;
+        dx[o + d] = (dy[o + d] * gate_act(g, o + d, swish) * w[h * D + d] - xhat * c1) * rstd;
       }
     }
 }

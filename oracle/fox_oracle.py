@@ -33,7 +33,10 @@ Reference lines restated here (paths relative to the reference checkout):
   (``group_norm_gated_ref`` here): per-group ``x / sqrt(mean(x^2) + eps) * weight``
   times ``sigmoid(g)`` (or ``g * sigmoid(g)``), evaluated in the upcast dtype.
   Pinned by ``torch.nn.functional.rms_norm`` per group, ``gradcheck`` in fp64 and
-  the C restatement.
+  the C restatement.  ``group_norm_ref`` is the same without a gate
+  (``layernorm.py:77-110``), pinned the same way; ``qk_norm_threshold_ref``
+  (``modeling_forgetting_transformer.py:371-380``) is pinned by the bound it
+  states: no logit of normalised q, k exceeds it (brute force).
 
 Pinned by (see tests/test_oracle_cpu.py): ``scaled_dot_product_attention`` with
 an additive mask, ``torch.logsumexp``, the ``g == 0`` and constant-``g``
@@ -50,6 +53,8 @@ import torch
 
 __all__ = [
     "group_norm_gated_ref",
+    "group_norm_ref",
+    "qk_norm_threshold_ref",
     "token_shift_ref",
     "cumulative_log_decay",
     "auto_threshold",
@@ -285,18 +290,43 @@ def token_shift_ref(x: torch.Tensor, prev_weight: torch.Tensor, curr_weight: tor
     return (x_prev * prev_weight[..., None] + x * curr_weight[..., None]).to(x.dtype)
 
 
-def group_norm_gated_ref(x: torch.Tensor, g: torch.Tensor, weight: torch.Tensor, num_groups: int, eps: float = 1e-6,
-                         activation: str = "sigmoid", upcast: bool = True) -> torch.Tensor:
+def group_norm_gated_ref(x: torch.Tensor, g: Optional[torch.Tensor], weight: torch.Tensor, num_groups: int,
+                         eps: float = 1e-6, activation: str = "sigmoid", upcast: bool = True) -> torch.Tensor:
     """Per-group RMS norm with weight, times the gate activation (reference
-    ``fuse_norm_gate.py:18-53`` with ``is_rms_norm=True``, no bias, no residual).  x, g: (..., G*D)."""
+    ``fuse_norm_gate.py:18-53`` with ``is_rms_norm=True``, no bias, no residual).  x, g: (..., G*D).
+    ``activation="none"`` (``g`` unused) is the plain per-group RMS norm of ``layernorm.py:77-110``."""
     dtype = x.dtype
     if upcast and dtype in (torch.float16, torch.bfloat16):
-        x, g, weight = x.float(), g.float(), weight.float()
+        x, weight = x.float(), weight.float()
+        g = g.float() if g is not None else None
     shape = x.shape
     xg = x.reshape(*shape[:-1], num_groups, shape[-1] // num_groups)
     wg = weight.reshape(num_groups, shape[-1] // num_groups)
     rstd = 1 / torch.sqrt(xg.square().mean(dim=-1, keepdim=True) + eps)
     out = (xg * rstd * wg).reshape(shape)
-    s = torch.sigmoid(g)
-    out = out * (s if activation == "sigmoid" else g * s)
+    if activation != "none":
+        s = torch.sigmoid(g)
+        out = out * (s if activation == "sigmoid" else g * s)
     return out.to(dtype)
+
+
+def group_norm_ref(x: torch.Tensor, weight: torch.Tensor, num_groups: int, eps: float = 1e-5,
+                   upcast: bool = True) -> torch.Tensor:
+    """Plain per-group RMS norm with weight (reference ``layernorm.py:77-110`` with ``is_rms_norm=True``, no
+    bias, no residual): what the FoX layer applies to queries and keys (``modeling_forgetting_transformer.py:
+    258-265, 314-325``)."""
+    return group_norm_gated_ref(x, None, weight, num_groups, eps, "none", upcast)
+
+
+def qk_norm_threshold_ref(q_norm_weight: torch.Tensor, k_norm_weight: torch.Tensor, num_heads: int, head_dim: int,
+                          seq_len: int, log_pruning_tolerance: float, share_param_across_head: bool = False) -> torch.Tensor:
+    """Pruning threshold from the QK-norm weights (``modeling_forgetting_transformer.py:371-380``): after an RMS
+    norm every query/key row has L2 norm at most ``max|w| * sqrt(D)``, so with ``sm_scale = 1/sqrt(D)`` the logits are
+    bounded by ``max|w_q| * max|w_k| * sqrt(D)``; the threshold is ``-(2 * bound + log T) + tolerance``, one per head
+    (a scalar when the heads share their weights)."""
+    if share_param_across_head:
+        bound = q_norm_weight.abs().max() * k_norm_weight.abs().max() * math.sqrt(head_dim)
+    else:
+        bound = (q_norm_weight.view(num_heads, head_dim).abs().max(dim=-1).values
+                 * k_norm_weight.view(num_heads, head_dim).abs().max(dim=-1).values * math.sqrt(head_dim))
+    return -(2 * bound + math.log(seq_len)) + log_pruning_tolerance

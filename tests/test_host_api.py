@@ -3,6 +3,7 @@ loads and exports every symbol the public header declares, argument validation i
 the C ABI returns error codes before anything is launched, and the Python wrapper
 raises the reference's error types (ops/forgetting_attention.py:78-137, 447-448)."""
 import ctypes as C
+import math
 import re
 
 import pytest
@@ -126,14 +127,19 @@ def test_norm_gate_c_abi_and_wrapper_checks():
     base = C.addressof(buf)
     base += (-base) % 16
 
-    def args(D=64, dtype=0, act=0, x=base, y=base + 1024, xs=64, rstd=base + 4096, weight=base + 2048):
-        return _lib.NormGateArgs(2, 1, D, dtype, act, 1e-6, x, xs, base + 512, 64, weight, y, 64, rstd,
+    def args(D=64, dtype=0, act=0, x=base, y=base + 1024, xs=64, rstd=base + 4096, weight=base + 2048, g=base + 512):
+        return _lib.NormGateArgs(2, 1, D, dtype, act, 1e-6, x, xs, g, 64, weight, y, 64, rstd,
                                  None, 0, None, 0, None, 0, None, None)
 
     assert lib.fox_norm_gate_fwd(C.byref(args(D=48)), None) == -1 and b"head dim" in lib.fox_last_error()
     assert lib.fox_norm_gate_fwd(C.byref(args(dtype=2)), None) == -1 and b"dtype" in lib.fox_last_error()
     assert lib.fox_norm_gate_fwd(C.byref(args(act=5)), None) == -1 and b"activation" in lib.fox_last_error()
     assert lib.fox_norm_gate_fwd(C.byref(args(x=None)), None) == -1
+    assert lib.fox_norm_gate_fwd(C.byref(args(g=None)), None) == -1 and b"g must not be NULL" in lib.fox_last_error()
+    # the plain norm (FOX_ACT_NONE) takes no gate, and is checked like the gated one otherwise
+    assert lib.fox_norm_gate_fwd(C.byref(args(act=2, g=None, y=None)), None) == -1 and b"y must not be NULL" in lib.fox_last_error()
+    assert lib.fox_norm_gate_fwd(C.byref(args(act=2, g=None, xs=60)), None) == -2
+    assert lib.fox_norm_gate_bwd(C.byref(args(act=2, g=None)), None) == -1      # dy, dx missing
     assert lib.fox_norm_gate_fwd(C.byref(args(y=None)), None) == -1 and b"y must not be NULL" in lib.fox_last_error()
     assert lib.fox_norm_gate_fwd(C.byref(args(x=base + 4)), None) == -2
     assert lib.fox_norm_gate_fwd(C.byref(args(xs=60)), None) == -2 and b"row strides" in lib.fox_last_error()
@@ -154,12 +160,41 @@ def test_norm_gate_c_abi_and_wrapper_checks():
         group_norm_gated(x, x, w, None, "sigmoid", residual=x, is_rms_norm=True, num_groups=2)
     with pytest.raises(ValueError):
         group_norm_gated(x, x, w, None, "tanh", is_rms_norm=True, num_groups=2)
-    with pytest.raises(AssertionError):
+    with pytest.raises(ValueError, match="divisible"):
         group_norm_gated(x, x, w, None, "sigmoid", is_rms_norm=True, num_groups=3)
     with pytest.raises(AssertionError):
         group_norm_gated(x.float(), x.float(), w, None, "sigmoid", is_rms_norm=True, num_groups=2)
     with pytest.raises(RuntimeError, match="no CPU path"):
         group_norm_gated(x, x, w, None, "sigmoid", is_rms_norm=True, num_groups=2)
+
+    from forgetting_transformer import group_norm, rms_norm
+    with pytest.raises(NotImplementedError):
+        group_norm(x, w, torch.zeros(128), is_rms_norm=True, num_groups=2)     # bias
+    with pytest.raises(NotImplementedError):
+        group_norm(x, w, None, is_rms_norm=False, num_groups=2)                # mean-centred norm
+    with pytest.raises(ValueError, match="divisible"):
+        group_norm(x, w, None, is_rms_norm=True, num_groups=3)                 # layernorm.py:723-724
+    with pytest.raises(AssertionError):
+        group_norm(x.float(), w, None, is_rms_norm=True, num_groups=2)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        rms_norm(x, w)
+
+
+def test_qk_norm_threshold_matches_the_layer_rule():
+    """modeling_forgetting_transformer.py:371-380, both weight-sharing modes."""
+    from forgetting_transformer import qk_norm_threshold
+    H, D, T, tol = 3, 16, 777, -12.0
+    gen = torch.Generator().manual_seed(3)
+    wq, wk = torch.randn(H * D, generator=gen), torch.randn(H * D, generator=gen)
+    thr = qk_norm_threshold(wq, wk, H, D, T, tol)
+    assert thr.shape == (H,) and thr.dtype == torch.float32 and not thr.requires_grad
+    for h in range(H):
+        want = -(2 * wq[h * D:(h + 1) * D].abs().max() * wk[h * D:(h + 1) * D].abs().max() * math.sqrt(D) + math.log(T)) + tol
+        assert torch.allclose(thr[h], want, rtol=1e-6)
+    thr0 = qk_norm_threshold(wq[:D], wk[:D], H, D, T, tol, share_param_across_head=True)
+    assert thr0.shape == () and torch.allclose(thr0, thr[0], rtol=1e-6)
+    with pytest.raises(AssertionError):
+        qk_norm_threshold(wq[:D], wk[:D], H, D, T, tol)                        # per-head weights expected (:376)
 
 
 def test_workspace_query():

@@ -405,3 +405,59 @@ def test_group_norm_gated_against_library_rms_norm_and_c(c_oracle, activation):
                                       C.c_int64(R), G, D, C.c_double(eps), swish)
     for got, ref in ((y_c, out), (dx_c, dx), (dg_c, dg), (dw_c, dw)):
         assert np.allclose(got, ref.detach().numpy(), rtol=1e-10, atol=1e-12)
+
+
+def test_group_norm_against_library_rms_norm_and_c(c_oracle):
+    """The plain (ungated) per-group RMS norm applied to queries and keys."""
+    R, G, D, eps = 9, 4, 8, 1e-5
+    gen = torch.Generator().manual_seed(14)
+    x = torch.randn(R, G * D, generator=gen, dtype=torch.float64)
+    w = torch.rand(G * D, generator=gen, dtype=torch.float64) + 0.5
+    out = O.group_norm_ref(x, w, G, eps)
+    want = torch.cat([F.rms_norm(x[:, h * D:(h + 1) * D], (D,), w[h * D:(h + 1) * D], eps) for h in range(G)], dim=1)
+    assert torch.allclose(out, want, rtol=1e-12, atol=1e-12)
+    # one group = the whole row: the textbook RMS norm
+    assert torch.allclose(O.group_norm_ref(x, w, 1, eps), F.rms_norm(x, (G * D,), w, eps), rtol=1e-12, atol=1e-12)
+    xr, wr = x.clone().requires_grad_(), w.clone().requires_grad_()
+    assert torch.autograd.gradcheck(lambda a, b: O.group_norm_ref(a, b, G, eps), (xr, wr), eps=1e-6, atol=1e-6)
+    dy = torch.randn(R, G * D, generator=gen, dtype=torch.float64)
+    dx, dw = torch.autograd.grad(O.group_norm_ref(xr, wr, G, eps), (xr, wr), dy)
+    xn, wn, dyn = (t.numpy().copy() for t in (x, w, dy))
+    y_c, dx_c, dw_c = np.empty_like(xn), np.empty_like(xn), np.empty_like(wn)
+    c_oracle.fox_oracle_norm_gate_fwd(_dptr(xn), None, _dptr(wn), _dptr(y_c), C.c_int64(R), G, D, C.c_double(eps), 2)
+    c_oracle.fox_oracle_norm_gate_bwd(_dptr(xn), None, _dptr(wn), _dptr(dyn), _dptr(dx_c), None, _dptr(dw_c),
+                                      C.c_int64(R), G, D, C.c_double(eps), 2)
+    for got, ref in ((y_c, out), (dx_c, dx), (dw_c, dw)):
+        assert np.allclose(got, ref.detach().numpy(), rtol=1e-10, atol=1e-12)
+
+
+@pytest.mark.parametrize("share", [False, True])
+def test_qk_norm_threshold_bounds_every_logit(share):
+    """The threshold is -(2*bound + log T) + tolerance where `bound` must dominate every |q.k|/sqrt(D) of
+    RMS-normalised rows (eps > 0 only shrinks them): brute force over random rows and adversarial ones."""
+    H, D, T, tol = 3, 16, 50, -7.5
+    gen = torch.Generator().manual_seed(15)
+    wq = torch.randn(D if share else H * D, generator=gen, dtype=torch.float64)
+    wk = torch.randn(D if share else H * D, generator=gen, dtype=torch.float64)
+    thr = O.qk_norm_threshold_ref(wq, wk, H, D, T, tol, share)
+    assert thr.shape == (() if share else (H,))
+    bound = (-(thr - tol) - math.log(T)) / 2
+    x = torch.randn(200, H * D, generator=gen, dtype=torch.float64) * 10
+    # adversarial rows: all the mass on the coordinate with the largest |w|
+    for h in range(H):
+        wqh = wq if share else wq[h * D:(h + 1) * D]
+        x[h, h * D:(h + 1) * D] = 0.0
+        x[h, h * D + int(wqh.abs().argmax())] = 5.0
+    wq_full = wq.repeat(H) if share else wq
+    wk_full = wk.repeat(H) if share else wk
+    qn = O.group_norm_ref(x, wq_full, H, 0.0).view(-1, H, D)
+    kn = O.group_norm_ref(x, wk_full, H, 0.0).view(-1, H, D)
+    logits = torch.einsum("ihd,jhd->hij", qn, kn) / math.sqrt(D)
+    worst = logits.abs().amax(dim=(1, 2))
+    assert (worst <= (bound if not share else bound.expand(H)) * (1 + 1e-12)).all()
+    # the closed form itself, head by head
+    for h in range(H):
+        a = (wq if share else wq[h * D:(h + 1) * D]).abs().max()
+        b = (wk if share else wk[h * D:(h + 1) * D]).abs().max()
+        want = -(2 * a * b * math.sqrt(D) + math.log(T)) + tol
+        assert torch.allclose(thr if share else thr[h], want, rtol=1e-14, atol=0)
