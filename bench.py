@@ -49,6 +49,9 @@ WORKLOADS = {
     # name: B, T(M), N, H, D, gate mean, gate std, head_first, fwd_only, seq_start
     "c2": dict(B=4, M=512, N=512, H=12, D=64, mean=0.0, std=1.0, head_first=False, fwd_only=False, pad=False),
     "c3": dict(B=4, M=16384, N=16384, H=16, D=128, mean=3.0, std=1.0, head_first=False, fwd_only=False, pad=False),
+    # config 3 at the head dim of the reference's own models (hidden_size / num_heads = 64 in every
+    # configs/experiment/longcrawl64/forgetting_transformer/*.yaml): same token count and matmul work, twice the heads
+    "c3d64": dict(B=4, M=16384, N=16384, H=32, D=64, mean=3.0, std=1.0, head_first=False, fwd_only=False, pad=False),
     "c4": dict(B=4, M=16384, N=16384, H=16, D=128, mean=-1.0, std=2.0, head_first=False, fwd_only=False, pad=False),
     "c5": dict(B=16, M=128, N=32768, H=16, D=128, mean=2.0, std=1.0, head_first=True, fwd_only=True, pad=True),
     # one new token against the same cache (the reference's M == 1 path, ops/forgetting_attention.py:148-153)

@@ -113,7 +113,12 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
                                           const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16],
                                           f32x16 (&dkacc)[(D + 31) / 32], f32x16 (&dvacc)[(D + 31) / 32], float& csum,
                                           float qk_scale, float colc, int lane, Dma dma) {
-  constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32, NCH = 8;
+  constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32;
+  // chunks per slot: as many as the larger of the two MFMA groups needs (one k-step of S and dP, one accumulation
+  // pair of dV and dK per chunk), so that every chunk carries matrix work; the 16 scores per lane of a block are
+  // dealt out evenly over them
+  constexpr int NCH = KK > 2 * DB ? KK : 2 * DB, SPC = 16 / NCH;
+  static_assert(16 % NCH == 0 && (SPC == 2 || SPC == 4 || SPC == 8), "whole scores per chunk, whole operands per 8 scores");
   constexpr int NC = (MB + 2) * NCH;  // chunks of the step: slots -1 .. MB
   constexpr int PF = 3;               // LDS operands are requested this many chunks before their MFMAs
   constexpr int kDmaEvery = (NC - NCH) / (NDMA > 0 ? NDMA : 1) > 0 ? (NC - NCH) / (NDMA > 0 ? NDMA : 1) : 1;
@@ -150,7 +155,7 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
     constexpr bool do_s = slot + 1 < MB, do_v = slot >= 0 && slot < MB, do_c = slot >= 1;
     constexpr int bs = slot + 1, bv = slot, bc = slot - 1;
     fetch(std::integral_constant<int, c + PF>{});
-    if constexpr (u == NCH - PF) init_block(bs + 1);
+    if constexpr (u == (NCH > PF ? NCH - PF : 0)) init_block(bs + 1);
     // the next tile's load instructions, one every kDmaEvery chunks from the second slot on
     if constexpr (c >= NCH && (c - NCH) % kDmaEvery == 0 && (c - NCH) / kDmaEvery < NDMA)
       dma(std::integral_constant<int, (c - NCH) / kDmaEvery>{});
@@ -164,17 +169,18 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
     }
     if constexpr (do_v) {
 #pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const int r = 2 * u + e;
+      for (int e = 0; e < SPC; ++e) {
+        const int r = SPC * u + e;
         const float p = __builtin_amdgcn_exp2f(fmaf(s[bv][r], qk_scale, -colc));
         const float ds = p * dp[bv][r];
         s[bv][r] = p;
         dp[bv][r] = ds;
         csum += ds;
       }
-      if constexpr (u % 4 == 3) {  // eight scores complete: pack one MFMA operand each of P and dS
-        pb[bv][u / 4] = pack8<Tr>(s[bv], 8 * (u / 4));
-        dsb[bv][u / 4] = pack8<Tr>(dp[bv], 8 * (u / 4));
+      if constexpr ((SPC * (u + 1)) % 8 == 0) {  // eight scores complete: pack one MFMA operand each of P and dS
+        constexpr int hh = SPC * (u + 1) / 8 - 1;
+        pb[bv][hh] = pack8<Tr>(s[bv], 8 * hh);
+        dsb[bv][hh] = pack8<Tr>(dp[bv], 8 * hh);
       }
     }
     constexpr int kMfmaMask = 0x008, kValuMask = 0x002, kTransMask = 0x400;
@@ -183,15 +189,15 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(kValuMask, 4, 0);
-        __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(kValuMask, 2 * SPC, 0);
+        __builtin_amdgcn_sched_group_barrier(kTransMask, SPC / 2, 0);
       }
     } else if constexpr (do_v && n_mfma == 2) {
 #pragma unroll
       for (int k = 0; k < 2; ++k) {
         __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(kValuMask, 8, 0);
-        __builtin_amdgcn_sched_group_barrier(kTransMask, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(kValuMask, 4 * SPC, 0);
+        __builtin_amdgcn_sched_group_barrier(kTransMask, SPC / 2, 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -199,7 +205,7 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
 }
 
 template <typename Tr, int D>
-__global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
+__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void dkdv_kernel(const BwdK a) {
   constexpr int BN = kKvBN, BMQ = kKvBM;
   constexpr int KK = D / 16, DB = (D + 31) / 32;
   static_assert(BN == 128, "four waves of 32 key rows");
@@ -328,6 +334,23 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     if (n_diag == 0) issue(m_top, q_tile0, do_tile0);
     if (row_lane) { rc_s0[row_slot] = rc_term(); dl_s0[row_slot] = dl_term(); }
   }
+  if constexpr (D <= 64) {
+    // Small head dims leave room for two workgroups per CU: the second wave on each SIMD fills the matrix pipe
+    // while the first does its vector work, so the plain step is used for interior tiles too.
+    for (int t = 0; t < n_int; ++t) {
+      const bool odd = t & 1;
+      wait_vmem_all();
+      __syncthreads();
+      if (t + 1 < n_int) issue(m_top - (t + 1) * BMQ, odd ? q_tile0 : q_tile1, odd ? do_tile0 : do_tile1);
+      const int ms = m_top - t * BMQ;
+      dkdv_step<Tr, D>(odd ? q_tile1 : q_tile0, odd ? do_tile1 : do_tile0, odd ? rc_s1 : rc_s0, odd ? dl_s1 : dl_s0, kreg, vreg,
+                       dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane);
+      if (t + 1 < n_int && row_lane) {
+        (odd ? rc_s0 : rc_s1)[row_slot] = rc_term();
+        (odd ? dl_s0 : dl_s1)[row_slot] = dl_term();
+      }
+    }
+  } else {
   constexpr int PER = DirectTileLoader<D, BMQ>::PER;
   for (int t = 0; t < n_int; t += 2) {
     wait_vmem_all();
@@ -363,6 +386,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdK a) {
     }
   }
 
+  }
   wait_vmem_all();  // whatever was requested last (possibly an empty tile) has landed before the buffers are reused
   const float ctot = half_sum(csum);
   if (n < N && g == 0) a.dc[(int64_t)bh * N + n] = -ctot;
