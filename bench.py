@@ -280,6 +280,30 @@ def prefill_report(steps, warmup):
             "frac_of_8TBps": (kv_bytes + other) / t * 1e-9 / PEAK_HBM_GBPS}
 
 
+def head_dim_report(steps, warmup):
+    """The headline step at head dim 64 (what every model configuration of the reference uses:
+    configs/experiment/longcrawl64/forgetting_transformer/*.yaml have hidden_size / num_heads = 64),
+    same token count and matmul work as the D = 128 workload."""
+    from forgetting_transformer import forgetting_attention
+
+    w = WORKLOADS["c3d64"]
+    tensors = synth(w, "cuda")
+    q, k, v, log_fgate, dout, _ = tensors
+    q, k, v, log_fgate = (x.requires_grad_() for x in (q, k, v, log_fgate))
+
+    def step():
+        forgetting_attention(q, k, v, log_fgate, head_first=w["head_first"]).backward(dout)
+        q.grad = k.grad = v.grad = log_fgate.grad = None
+    t = time_steps(step, steps, warmup)
+    st = stage_times(w, tensors, max(3, steps))
+    unit = flops_fwd(w) / 2.0
+    rep = {"workload": f"B{w['B']} T{w['M']} H{w['H']} D{w['D']} bf16 fwd+bwd, gate logits N({w['mean']},{w['std']}), no pruning",
+           "ms_per_step": t * 1e3, "tflops": 7 * unit / t * 1e-12, "frac_of_bf16_peak": 7 * unit / t * 1e-12 / PEAK_BF16_TFLOPS,
+           "kernels": {name: {"ms": st[name] * 1e3, "tflops": m * unit / st[name] * 1e-12}
+                       for name, m in (("fwd", 2), ("bwd_dkdv", 4), ("bwd_dq", 3))}}
+    return rep
+
+
 def shift_report(ns):
     """Token shift (the key/value pre-processing of the FoX layer) at the training-layer shape:
     forward + backward, HBM-bound; one JSON line of its own."""
@@ -487,6 +511,8 @@ def main():
         line["acp"] = acp_report(max(2, ns.steps // 2), 1)
         torch.cuda.empty_cache()
         line["prefill"] = prefill_report(max(5, ns.steps), 2)
+        torch.cuda.empty_cache()
+        line["head_dim_64"] = head_dim_report(max(2, ns.steps // 2), 1)
     print(json.dumps(line))
 
 

@@ -407,7 +407,11 @@ __device__ __forceinline__ void dq_tile(const char* k_tile, const char* v_tile, 
                                int a_w0, float qk_scale, float rowc, float delta, int lane) {
   constexpr int BN = kFwdBN, KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
   const int g = lane >> 5, i = lane & 31;
-  const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  // dP starts from -delta (constant along a query row, i.e. per lane) instead of zero: the matrix pipe does the
+  // subtraction.  The sixteen equal registers are loop-invariant for the caller.
+  f32x16 neg_delta;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) neg_delta[r] = -delta;
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     const int nb0 = n0 + 32 * nb;
@@ -415,7 +419,7 @@ __device__ __forceinline__ void dq_tile(const char* k_tile, const char* v_tile, 
     f32x16 s = acc_init(cn_s, 32 * nb, g);
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) s = Tr::mfma32(lds_row_operand<D>(k_tile, 32 * nb + i, 2 * kk + g), qreg[kk], s);
-    f32x16 dp = Tr::mfma32(lds_row_operand<D>(v_tile, 32 * nb + i, g), doreg[0], zero);
+    f32x16 dp = Tr::mfma32(lds_row_operand<D>(v_tile, 32 * nb + i, g), doreg[0], neg_delta);
 #pragma unroll
     for (int kk = 1; kk < KK; ++kk) dp = Tr::mfma32(lds_row_operand<D>(v_tile, 32 * nb + i, 2 * kk + g), doreg[kk], dp);
 #pragma unroll
@@ -426,7 +430,7 @@ __device__ __forceinline__ void dq_tile(const char* k_tile, const char* v_tile, 
     }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float ds = s[r] * (dp[r] - delta);
+      const float ds = s[r] * dp[r];
       dp[r] = ds;
       rsum += ds;
     }
