@@ -357,6 +357,23 @@ def test_random_configurations(fa, case):
         assert rel_err(x, r) <= tol, (name, case, rel_err(x, r), tol, dict(B=B, H=H, M=M, N=N, D=D, thr=thr_kind))
 
 
+@pytest.mark.parametrize("D", [16, 32, 64])
+@pytest.mark.parametrize("M,N,seq,thr", [(4100, 4100, None, None), (3000, 4500, [700], None), (4096, 4096, None, -6.0)])
+def test_long_sequences_at_small_head_dims(fa, D, M, N, seq, thr):
+    """Dozens of interior steps per key tile (both tile buffers in turn, with tails) on the dK/dV path that head dims
+    <= 64 take (two workgroups per CU, plain step for every tile)."""
+    q, k, v, g, do, ss = make_inputs(1, 2, M, N, D, device="cuda", head_first=True, seq_start=seq, seed=40 + D,
+                                     gate_mean=4.0, gate_std=1.0)
+    ref = O.forgetting_attention_ref_grads(q, k, v, g, do, head_first=True, seq_start=ss, bh_chunk=1)
+    q, k, v, g = (x.requires_grad_() for x in (q, k, v, g))
+    out = fa(q, k, v, g, head_first=True, seq_start=ss, adaptive_threshold=thr)
+    out.backward(do)
+    tol = REL_TOL + (4.0 * N * math.exp(thr) if thr is not None else 0.0)
+    for name, x, r in zip(("out", "dq", "dk", "dv", "dlog_fgate"), (out, q.grad, k.grad, v.grad, g.grad), ref):
+        assert torch.isfinite(x).all(), name
+        assert rel_err(x, r) <= tol, (name, rel_err(x, r), tol)
+
+
 # --------------------------------------------------------------------------------------
 # benchmark configurations 3-5 at full size
 # --------------------------------------------------------------------------------------
