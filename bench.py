@@ -43,7 +43,7 @@ PEAK_HBM_GBPS = 8000.0
 # passes over this script (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
 # plain 1 GiB copies of --copy-calibration (fetch x2.00, write x1.00); profiles/hbm_traffic_c3_c5.md.
 # Counters cannot be read from inside the timed run, so the figure is carried here.
-MEASURED_TRAFFIC_BYTES = {"c3": (2.049 + 0.504) * 2**30, "c5": (3.442 + 0.032) * 2**30, "decode": 3.568 * 2**30}
+MEASURED_TRAFFIC_BYTES = {"c3": (2.049 + 0.504) * 2**30, "c5": (3.442 + 0.032) * 2**30, "decode": (3.565 + 0.001) * 2**30}
 
 WORKLOADS = {
     # name: B, T(M), N, H, D, gate mean, gate std, head_first, fwd_only, seq_start

@@ -512,36 +512,49 @@ FOX_INSTANTIATE_FWD(Bf16)
 FOX_INSTANTIATE_FWD(Fp16)
 
 template <typename Tr, int D>
-static hipError_t launch_fwd_d(const FwdK& a, hipStream_t s) {
-  if (a.splits <= 1) {
+static hipError_t launch_fwd_d(const FwdK& a, int dtype, hipStream_t s) {
+  if (a.M == 1) {  // decode step: the streaming kernel, one workgroup per (batch, head, key split)
+    const hipError_t e = launch_fwd_decode(a, D, dtype, s);
+    if (e != hipSuccess || a.splits <= 1) return e;
+  } else if (a.splits <= 1) {
     hipLaunchKernelGGL((fwd_kernel<Tr, D, false>), dim3((unsigned)(a.n_mtiles * a.B * a.H)), dim3(256), 0, s, a);
     return hipGetLastError();
+  } else {
+    hipLaunchKernelGGL((fwd_kernel<Tr, D, true>), dim3((unsigned)(a.n_mtiles * a.splits * a.B * a.H)), dim3(256), 0, s, a);
   }
-  hipLaunchKernelGGL((fwd_kernel<Tr, D, true>), dim3((unsigned)(a.n_mtiles * a.splits * a.B * a.H)), dim3(256), 0, s, a);
   const int64_t threads = (int64_t)a.B * a.H * a.M * (D / 4);
   hipLaunchKernelGGL((combine_kernel<Tr, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, a);
   return hipGetLastError();
 }
 
 template <typename Tr>
-static hipError_t launch_fwd_t(const FwdK& a, int D, hipStream_t s) {
+static hipError_t launch_fwd_t(const FwdK& a, int D, int dtype, hipStream_t s) {
   switch (D) {
-    case 16: return launch_fwd_d<Tr, 16>(a, s);
-    case 32: return launch_fwd_d<Tr, 32>(a, s);
-    case 64: return launch_fwd_d<Tr, 64>(a, s);
-    case 128: return launch_fwd_d<Tr, 128>(a, s);
+    case 16: return launch_fwd_d<Tr, 16>(a, dtype, s);
+    case 32: return launch_fwd_d<Tr, 32>(a, dtype, s);
+    case 64: return launch_fwd_d<Tr, 64>(a, dtype, s);
+    case 128: return launch_fwd_d<Tr, 128>(a, dtype, s);
     default: return hipErrorInvalidValue;
   }
 }
 
 hipError_t launch_fwd(const FwdK& a, int D, int dtype, hipStream_t s) {
-  return dtype == 0 ? launch_fwd_t<Bf16>(a, D, s) : launch_fwd_t<Fp16>(a, D, s);
+  return dtype == 0 ? launch_fwd_t<Bf16>(a, D, dtype, s) : launch_fwd_t<Fp16>(a, D, dtype, s);
 }
 
 // Number of key splits the forward uses for a shape: 1 unless the grid of query tiles
 // alone leaves most of the chip idle while each workgroup has a long key loop (chunked
-// prefill, decode).  Splits are sized to give every CU about two workgroups.
+// prefill, decode).  Splits are sized to give every CU about two workgroups; the streaming
+// kernel of the single-query case keeps no tile in LDS and takes about eight per CU, at
+// least 512 keys each.
 int fwd_key_splits(int B, int H, int M, int N) {
+  if (M == 1) {
+    const int64_t bh = (int64_t)B * H;
+    int64_t splits = (2048 + bh - 1) / bh;
+    splits = splits > N / 512 ? N / 512 : splits;
+    splits = splits > 64 ? 64 : splits;
+    return splits < 1 ? 1 : (int)splits;
+  }
   const int64_t wgs = (int64_t)((M + kFwdBM - 1) / kFwdBM) * B * H;
   const int key_tiles = (N + kFwdBN - 1) / kFwdBN;
   if (wgs >= 512 || key_tiles < 16) return 1;

@@ -84,6 +84,7 @@ int fwd_key_splits(int B, int H, int M, int N);
 hipError_t launch_bwd_delta(const BwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_bwd_dkdv(const BwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_bwd_dq(const BwdK& a, int D, int dtype, hipStream_t s);
+hipError_t launch_fwd_decode(const FwdK& a, int D, int dtype, hipStream_t s);  // M == 1, without the merge of the splits
 hipError_t launch_norm_gate(const NormGateK& a, int D, int dtype, bool bwd, int act, hipStream_t s);  // act: FOX_ACT_*
 int64_t norm_gate_strips(int64_t rows);
 int64_t norm_gate_workspace_rows(int64_t rows);

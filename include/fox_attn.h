@@ -114,7 +114,8 @@ typedef struct fox_fwd_args {
 /*
  * Forward: o = softmax(q k^T sm_scale + c_i - c_j over seq_start <= j <= i+N-M) v.
  * Replaces _find_start_index_kernel (:695-745) + _fwd_kernel (:505-693) as launched
- * by ForgettingAttention.forward (:159-204).
+ * by ForgettingAttention.forward (:159-204).  M == 1 (one new token against the cache) takes a
+ * dot-free streaming kernel, like the reference's BLOCK_M = 1 case (:148-153, :637-641, :665-668).
  */
 int fox_attn_fwd(const fox_fwd_args* args, void* stream);
 

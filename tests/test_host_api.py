@@ -205,6 +205,11 @@ def test_workspace_query():
     assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(16, 16, 128, 32768, 128, 0)), C.byref(need)) == 0
     assert need.value > 0 and need.value % (16 * 16 * 128 * 130 * 4) == 0   # splits x rows x (D + 2) floats
     assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(1, 1, 1, 100, 64, 0)), C.byref(need)) == 0 and need.value == 0
+    # one query row against a long cache: the streaming kernel takes 2048 / (B*H) splits of at least 512 keys
+    assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(16, 16, 1, 32768, 128, 0)), C.byref(need)) == 0
+    assert need.value == 8 * 16 * 16 * 130 * 4
+    assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(1, 2, 1, 2048, 64, 0)), C.byref(need)) == 0
+    assert need.value == 4 * 1 * 2 * 66 * 4
     assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(1, 1, 1, 100, 48, 0)), C.byref(need)) == -1
     assert lib.fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(1, 1, 1, 100, 64, 0)), None) == -1
 
