@@ -165,6 +165,39 @@ def test_key_split_shapes(fa, B, H, M, N, D, seq, thr):
     run_case(fa, B, H, M, N, D, seq_start=seq, thr=thr, seed=N, gate_mean=4.0, gate_std=1.0)
 
 
+@pytest.mark.parametrize("D", [16, 32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,head_first,seq,thr", [
+    (1, True, None, None), (37, False, None, None), (300, True, [0, 299, 300], None),     # one workgroup per (b, h)
+    (5000, False, [17, 4999, 2500], None), (8192, True, None, -8.0), (6001, True, [100, 0, 6000], "auto")])  # key splits
+def test_single_query_streaming_kernel(fa, D, dtype, N, head_first, seq, thr):
+    """M = 1 (a decode step) runs through the dot-free streaming kernel: every head dim and dtype, both layouts,
+    with and without key splits, tails of the 4-wave rounds, left padding up to a fully padded row (o = 0,
+    zero gradients), pruning thresholds."""
+    B = 3 if seq is not None else 2
+    tol = REL_TOL if dtype == torch.bfloat16 else 1e-2
+    if isinstance(thr, float):
+        tol = tol + 4.0 * N * math.exp(thr)
+    run_case(fa, B, 2, 1, N, D, dtype=dtype, head_first=head_first, seq_start=seq, thr=thr, tol=tol, seed=N + D,
+             gate_mean=3.0, gate_std=1.5, qkv_std=0.8)
+
+
+def test_single_query_matches_last_row_of_a_full_forward(fa):
+    """The decode kernel against the tiled kernel itself: out and lse of the last query row of an M = N call, and the
+    first key block the pruning bound keeps (in keys, a multiple of the 64-key block)."""
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    B, H, N, D = 2, 3, 3000, 64
+    q, k, v, g, _, _ = make_inputs(B, H, N, N, D, device="cuda", head_first=True, seed=77, gate_mean=1.0, gate_std=2.0)
+    for thr in (None, -5.0):
+        full, lse_full, start_full = ForgettingAttention.apply(q, k, v, g, None, True, None, thr, True, True)
+        one, lse_one, start_one = ForgettingAttention.apply(q[:, :, -1:], k, v, g, None, True, None, thr, True, True)
+        assert rel_err(one, full[:, :, -1:]) <= 2.0 ** -7            # both round to bf16 once
+        assert torch.allclose(lse_one, lse_full[:, :, -1:], rtol=0, atol=2e-3)
+        # the bound of the last 128-row block is taken at its first row, the single row's at itself: never earlier
+        assert (start_one[:, :, 0] >= start_full[:, :, -1]).all() and (start_one % 64 == 0).all()
+        assert (start_one[:, :, 0] > 0).all() == (thr is not None)
+
+
 @pytest.mark.parametrize("sm_scale", [None, 0.5, 1.3])
 def test_sm_scale(fa, sm_scale):
     run_case(fa, 1, 2, 260, 260, 64, sm_scale=sm_scale, qkv_std=0.5, seed=3)
