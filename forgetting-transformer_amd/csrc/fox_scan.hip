@@ -18,29 +18,37 @@ constexpr int kScanThreads = 1024;  // one workgroup per row: few rows, long row
 
 // Scan of one row: element idx is produced by load(idx) and the running sum up to and including
 // it is handed to store(idx, sum).  REVERSE walks the row from its last element to its first.
+// A span of 8 x 1024 elements moves between memory and LDS with consecutive lanes on consecutive
+// elements (whole cache lines per wave instruction, whatever the caller's stride), and between LDS and
+// registers with eight consecutive elements per thread, the order the scan wants.
 template <bool REVERSE, typename Load, typename Store>
 __device__ __forceinline__ void scan_row(int N, Load load, Store store) {
   constexpr int PER = 8, NT = kScanThreads, SPAN = PER * NT;
   __shared__ double wave_tot[NT / kWave];
+  __shared__ __align__(16) float stage[SPAN];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   double carry = 0.0;
   float x[PER], x_next[PER];
-  auto fetch = [&](int base, float (&dst)[PER]) {  // the elements this thread owns in the span starting at base
+  auto fetch = [&](int base, float (&dst)[PER]) {  // element e of a thread sits at position base + e*NT + tid of the scan order
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
-      const int pos = base + tid * PER + e;            // position in scan order
-      const int idx = REVERSE ? N - 1 - pos : pos;     // element index
+      const int pos = base + e * NT + tid;
+      const int idx = REVERSE ? N - 1 - pos : pos;
       dst[e] = pos < N ? load(idx) : 0.f;
     }
   };
   fetch(0, x);
   for (int base = 0; base < N; base += SPAN) {
+#pragma unroll
+    for (int e = 0; e < PER; ++e) stage[e * NT + tid] = x[e];
     if (base + SPAN < N) fetch(base + SPAN, x_next);   // in flight while this span is scanned
+    __syncthreads();
+    const f32x4 lo4 = *reinterpret_cast<const f32x4*>(stage + tid * PER), hi4 = *reinterpret_cast<const f32x4*>(stage + tid * PER + 4);
     double v[PER];
     double run = 0.0;
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
-      run += (double)x[e];
+      run += (double)(e < 4 ? lo4[e & 3] : hi4[e & 3]);
       v[e] = run;
     }
     // inclusive scan of the per-thread totals across the wave, then across waves
@@ -60,16 +68,25 @@ __device__ __forceinline__ void scan_row(int N, Load load, Store store) {
       total += t;
     }
     before += incl - run;
+    f32x4 o_lo, o_hi;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      o_lo[e] = (float)(before + v[e]);
+      o_hi[e] = (float)(before + v[4 + e]);
+    }
+    *reinterpret_cast<f32x4*>(stage + tid * PER) = o_lo;   // each thread overwrites the eight values it read
+    *reinterpret_cast<f32x4*>(stage + tid * PER + 4) = o_hi;
+    carry += total;
+    __syncthreads();
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
-      const int pos = base + tid * PER + e;
+      const int pos = base + e * NT + tid;
       const int idx = REVERSE ? N - 1 - pos : pos;
-      if (pos < N) store(idx, (float)(before + v[e]));
+      if (pos < N) store(idx, stage[e * NT + tid]);
     }
-    carry += total;
 #pragma unroll
     for (int e = 0; e < PER; ++e) x[e] = x_next[e];
-    __syncthreads();
+    __syncthreads();  // the span has left LDS before the next one is written
   }
 }
 
