@@ -238,17 +238,23 @@ __global__ __launch_bounds__(256) void norm_max_kernel(View q, View k, int H, in
   const uint16_t* p = t.ptr + b * t.sb + h * t.sh;
   const int ch = tid % LPR;
   float best = 0.f;
-  for (int pass = 0; pass < ROWS / RPP; ++pass) {
-    const int row = blockIdx.x * ROWS + pass * RPP + tid / LPR;
-    float acc = 0.f;
-    if (row < T) {
-      const u32x4 x = *reinterpret_cast<const u32x4*>(p + (int64_t)row * t.st + ch * 8);
+  constexpr int U = (ROWS / RPP) < 8 ? (ROWS / RPP) : 8;  // rows in flight per thread
+  for (int pass = 0; pass < ROWS / RPP; pass += U) {
+    u32x4 x[U];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc += Tr::lo(x[e]) * Tr::lo(x[e]) + Tr::hi(x[e]) * Tr::hi(x[e]);
+    for (int u = 0; u < U; ++u) {
+      const int row = min(blockIdx.x * ROWS + (pass + u) * RPP + tid / LPR, T - 1);  // rows past the end repeat the last one
+      x[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (int64_t)row * t.st + ch * 8));
     }
 #pragma unroll
-    for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-    best = fmaxf(best, round16<Tr>(sqrtf(acc)));
+    for (int u = 0; u < U; ++u) {
+      float acc = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc += Tr::lo(x[u][e]) * Tr::lo(x[u][e]) + Tr::hi(x[u][e]) * Tr::hi(x[u][e]);
+#pragma unroll
+      for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+      best = fmaxf(best, round16<Tr>(sqrtf(acc)));
+    }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) best = fmaxf(best, __shfl_xor(best, off));

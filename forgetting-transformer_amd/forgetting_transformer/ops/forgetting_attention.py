@@ -129,6 +129,9 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
                 'adaptive_threshold must be either the string "auto", a float, or a Tensor, '
                 f"but got {adaptive_threshold}.")
             auto_threshold = True
+        elif isinstance(adaptive_threshold, (int, float)):
+            # same values as as_tensor + broadcast_to below, filled on the device: no host-to-device copy to wait for
+            adaptive_threshold = torch.full((B, H), float(adaptive_threshold), dtype=torch.float, device=q.device)
         else:
             adaptive_threshold = torch.as_tensor(adaptive_threshold, dtype=torch.float, device=q.device)
             try:
