@@ -207,6 +207,27 @@ def cpu_baseline(budget_s=10.0):
     }
 
 
+def graph_time(step, steps):
+    """Seconds per step of `step` captured once into a HIP graph and replayed: the same kernels without the host
+    between them (allocation, Python, launch latency), which matters when the whole step is about a millisecond."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up off the capture stream, as autograd under capture requires
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
 def kept_fraction(start_index, M, N, block_m, block_n):
     """Share of causal (query block, key block) tiles the forward visits, from the kernel's own bounds."""
     p_seq = N - M
@@ -236,17 +257,19 @@ def acp_report(steps, warmup):
             out.backward(dout)
             q.grad = k.grad = v.grad = log_fgate.grad = None
         t = time_steps(step, steps, warmup)
+        t_graph = graph_time(step, max(steps, 10))
         with torch.no_grad():
             out = forgetting_attention(q, k, v, log_fgate, adaptive_threshold=thr)
-        entry = {"ms_per_step": t * 1e3}
+        entry = {"ms_per_step": t * 1e3, "graph_replay_ms_per_step": t_graph * 1e3}
         if thr is None:
-            base, ref_out = t, out
+            base, base_graph, ref_out = t, t_graph, out
         else:
             with torch.no_grad():
                 _, _, si = ForgettingAttention.apply(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
                                                      log_fgate.transpose(1, 2), None, True, None, thr, False, True)
             kept = kept_fraction(si, w["M"], w["N"], block_m, block_n)
             entry.update(pruned_tile_fraction=1.0 - kept, speedup_vs_none=base / t,
+                         graph_replay_speedup_vs_none=base_graph / t_graph,
                          max_abs_diff_vs_none=(out.float() - ref_out.float()).abs().max().item())
         rep[name] = entry
     # where the pruned step spends its time: every kernel alone at threshold -10, against the bytes it must move
