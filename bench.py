@@ -303,6 +303,29 @@ def prefill_report(steps, warmup):
             "frac_of_8TBps": (kv_bytes + other) / t * 1e-9 / PEAK_HBM_GBPS}
 
 
+def decode_report(steps, warmup):
+    """One new token against the config-5 cache (M = 1): the streaming kernel, HBM-bound."""
+    from forgetting_transformer import forgetting_attention
+
+    w = WORKLOADS["decode"]
+    sets = [synth(w, "cuda", seed=20 + i) for i in range(3)]  # rotate so K/V do not sit in cache
+    idx = [0]
+
+    def step():
+        q, k, v, log_fgate, _, ss = sets[idx[0] % len(sets)]
+        idx[0] += 1
+        with torch.no_grad():
+            forgetting_attention(q, k, v, log_fgate, head_first=True, seq_start=ss)
+    t = time_steps(step, steps, warmup)
+    st = stage_times(w, sets[0], max(5, steps))
+    B, H, M, N, D = w["B"], w["H"], w["M"], w["N"], w["D"]
+    pad = sets[0][5].float()
+    alg = (2.0 * H * (N - pad) * D * 2).sum().item() + 2 * B * H * M * D * 2 + B * H * N * 4
+    return {"workload": "B16 M1 N32768 H16 D128 bf16 forward, head_first, seq_start~U[0,8192)",
+            "ms_per_step": t * 1e3, "kernel_ms": st["fwd"] * 1e3, "algorithmic_bytes": alg,
+            "kernel_hbm_gbps": alg / st["fwd"] * 1e-9, "kernel_frac_of_8TBps": alg / st["fwd"] * 1e-9 / PEAK_HBM_GBPS}
+
+
 def head_dim_report(steps, warmup):
     """The headline step at head dim 64 (what every model configuration of the reference uses:
     configs/experiment/longcrawl64/forgetting_transformer/*.yaml have hidden_size / num_heads = 64),
@@ -534,6 +557,8 @@ def main():
         line["acp"] = acp_report(max(2, ns.steps // 2), 1)
         torch.cuda.empty_cache()
         line["prefill"] = prefill_report(max(5, ns.steps), 2)
+        torch.cuda.empty_cache()
+        line["decode"] = decode_report(max(5, ns.steps), 2)
         torch.cuda.empty_cache()
         line["head_dim_64"] = head_dim_report(max(2, ns.steps // 2), 1)
     print(json.dumps(line))
