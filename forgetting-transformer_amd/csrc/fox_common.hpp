@@ -207,8 +207,11 @@ struct DirectTileLoader {
   }
   // Byte extent of the tile whose first row is row0, for its buffer resource: rows at or beyond row_limit
   // are out of range, and an extent of 0 (row_limit <= row0) makes every load return zero.
+  // Only the tile's own ROWS rows count, so the extent stays far below the 32-bit limit of a buffer resource
+  // however long the sequence and however large the row stride.
   __device__ __forceinline__ int extent(int64_t row_stride, int row0, int row_limit) const {
-    return row_limit > row0 ? (int)(((int64_t)(row_limit - 1 - row0) * row_stride + D) * 2) : 0;
+    const int rows = row_limit - row0 < ROWS ? row_limit - row0 : ROWS;
+    return rows > 0 ? (int)(((int64_t)(rows - 1) * row_stride + D) * 2) : 0;
   }
   // The j-th (a constant at every call site) of this wave's PER load instructions of the tile that
   // starts at p, so that a kernel can spread them over its compute instead of issuing them back to back
