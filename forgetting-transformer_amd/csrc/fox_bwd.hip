@@ -32,16 +32,21 @@ __global__ __launch_bounds__(256) void delta_kernel(const BwdK a) {
   const uint16_t* op = a.o.ptr + b * a.o.sb + h * a.o.sh;
   const uint16_t* dop = a.d_o.ptr + b * a.d_o.sb + h * a.d_o.sh;
   const int ch = tid % LPR;
+  // every load of the workgroup's rows is requested before the first one is used (rows past the end repeat the last row)
+  constexpr int NP = ROWS / RPP;
+  u32x4 x[NP], y[NP];
 #pragma unroll
-  for (int pass = 0; pass < ROWS / RPP; ++pass) {
+  for (int pass = 0; pass < NP; ++pass) {
+    const int m = min(blockIdx.x * ROWS + pass * RPP + tid / LPR, a.M - 1);
+    x[pass] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(op + (int64_t)m * a.o.st + ch * 8));
+    y[pass] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(dop + (int64_t)m * a.d_o.st + ch * 8));
+  }
+#pragma unroll
+  for (int pass = 0; pass < NP; ++pass) {
     const int m = blockIdx.x * ROWS + pass * RPP + tid / LPR;
     float acc = 0.f;
-    if (m < a.M) {
-      const u32x4 x = *reinterpret_cast<const u32x4*>(op + (int64_t)m * a.o.st + ch * 8);
-      const u32x4 y = *reinterpret_cast<const u32x4*>(dop + (int64_t)m * a.d_o.st + ch * 8);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc += Tr::lo(x[e]) * Tr::lo(y[e]) + Tr::hi(x[e]) * Tr::hi(y[e]);
-    }
+    for (int e = 0; e < 4; ++e) acc += Tr::lo(x[pass][e]) * Tr::lo(y[pass][e]) + Tr::hi(x[pass][e]) * Tr::hi(y[pass][e]);
 #pragma unroll
     for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
     if (m < a.M && ch == 0) a.delta[(int64_t)bh * a.M + m] = acc;
