@@ -148,7 +148,7 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, (SPC / 2 + NB - 1) / NB, 0);  // the chunk's v_max3 dealt out over its MFMAs
     }
     __builtin_amdgcn_sched_barrier(0);
   });
@@ -192,10 +192,10 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
     }
     if (c >= 1 && c < NSL) {
 #pragma unroll
-      for (int k = 0; k < DB; ++k) {
+      for (int k = 0; k < DB; ++k) {  // a slice has 20 vector and 8 exp instructions: dealt out over its DB MFMAs
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
-        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 20 / DB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x400, 8 / DB, 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
