@@ -7,7 +7,16 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "fox_kernels.hpp"
+
+// Library-owned scratch of fox_attn_fwd_noalloc: the partial (max, sum, accumulator) results of a key-split
+// forward.  Every GPU the library runs on holds its own copy of this array, at its own address, until the
+// process ends.  In host code the name is only a handle for hipGetSymbolAddress; kernels and copies get the
+// per-device address that call returns.
+#define FOX_NOALLOC_SCRATCH_BYTES (64ll << 20)
+static __device__ __align__(256) unsigned char scratch[FOX_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 
@@ -47,6 +56,27 @@ int check_view(const fox_view* v, const char* name) {
 int check_extent(const fox_view* v, int rows, int D, const char* name) {
   const int64_t bytes = ((int64_t)(rows - 1) * v->stride_t + D) * 2;
   if (v->stride_t <= 0 || bytes >= (int64_t)1 << 31) return fail(FOX_E_ARG, "%s: one (batch, head) slice must span less than 2 GiB with a positive row stride", name);
+  return FOX_OK;
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int scratch_of_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(FOX_E_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(FOX_E_ARG, "device index %d is outside the scratch table (0..%d)", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return fail(FOX_E_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
   return FOX_OK;
 }
 
@@ -155,6 +185,45 @@ int make_norm_gate(const fox_norm_gate_args* a, fox::NormGateK& k, bool bwd) {
   return FOX_OK;
 }
 
+// The forward with its key-split scratch passed separately: the caller's workspace (fox_attn_fwd) or the
+// library's own array (fox_attn_fwd_noalloc).  workspace == NULL never splits keys.
+int fwd_impl(const fox_fwd_args* args, void* workspace, int64_t workspace_bytes, void* stream, const char* what) {
+  FOX_TRY(check_dims(&args->dims));
+  FOX_TRY(check_view(&args->q, "q"));
+  FOX_TRY(check_view(&args->k, "k"));
+  FOX_TRY(check_view(&args->v, "v"));
+  FOX_TRY(check_view(&args->o, "o"));
+  FOX_TRY(check_extent(&args->k, args->dims.N, args->dims.D, "k"));
+  FOX_TRY(check_extent(&args->v, args->dims.N, args->dims.D, "v"));
+  if (!args->log_lambda || !args->lse) return fail(FOX_E_ARG, "log_lambda and lse must not be NULL");
+  fox::FwdK k{};
+  k.q = to_view(args->q);
+  k.k = to_view(args->k);
+  k.v = to_view(args->v);
+  k.o = to_view(args->o);
+  k.c = args->log_lambda;
+  k.lse = args->lse;
+  k.seq_start = args->seq_start;
+  k.thr = args->threshold;
+  k.first_block = args->first_block;
+  k.B = args->dims.B; k.H = args->dims.H; k.M = args->dims.M; k.N = args->dims.N;
+  k.sm_scale = args->sm_scale;
+  k.n_mtiles = (args->dims.M + fox::kFwdBM - 1) / fox::kFwdBM;
+  k.splits = 1;
+  if (workspace) {
+    const int splits = fox::fwd_key_splits(k.B, k.H, k.M, k.N);
+    const int64_t need = splits <= 1 ? 0 : (int64_t)splits * k.B * k.H * k.M * (args->dims.D + 2) * (int64_t)sizeof(float);
+    if (need > 0) {
+      if (workspace_bytes < need) return fail(FOX_E_ARG, "workspace too small: %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
+      if (((uintptr_t)workspace & 15) != 0) return fail(FOX_E_ALIGN, "workspace must be 16-byte aligned");
+      k.splits = splits;
+      k.ws_o = (float*)workspace;
+      k.ws_ml = k.ws_o + (int64_t)k.splits * k.B * k.H * k.M * args->dims.D;
+    }
+  }
+  return check_hip(fox::launch_fwd(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), what);
+}
+
 }  // namespace
 
 extern "C" {
@@ -239,13 +308,13 @@ int fox_cumsum_bwd(const float* dc, float* dg, int32_t B, int32_t H, int32_t N, 
 }
 
 int fox_auto_threshold(const fox_dims* dims, const fox_view* q, const fox_view* k, float sm_scale, float* thr,
-                       uint32_t* scratch, void* stream) {
+                       uint32_t* norm_scratch, void* stream) {
   FOX_TRY(check_dims(dims));
   FOX_TRY(check_view(q, "q"));
   FOX_TRY(check_view(k, "k"));
-  if (!thr || !scratch) return fail(FOX_E_ARG, "thr and scratch must not be NULL");
+  if (!thr || !norm_scratch) return fail(FOX_E_ARG, "thr and norm_scratch must not be NULL");
   return check_hip(fox::launch_auto_threshold(to_view(*q), to_view(*k), dims->B, dims->H, dims->M, dims->N, dims->D,
-                                              dims->dtype, sm_scale, thr, scratch, (hipStream_t)stream),
+                                              dims->dtype, sm_scale, thr, norm_scratch, (hipStream_t)stream),
                    "fox_auto_threshold");
 }
 
@@ -259,40 +328,20 @@ int fox_attn_fwd_workspace_bytes(const fox_dims* dims, int64_t* bytes) {
 
 int fox_attn_fwd(const fox_fwd_args* args, void* stream) {
   if (!args) return fail(FOX_E_ARG, "args is NULL");
+  return fwd_impl(args, args->workspace, args->workspace_bytes, stream, "fox_attn_fwd");
+}
+
+int fox_attn_fwd_noalloc(const fox_fwd_args* args, void* stream) {
+  if (!args) return fail(FOX_E_ARG, "args is NULL");
   FOX_TRY(check_dims(&args->dims));
-  FOX_TRY(check_view(&args->q, "q"));
-  FOX_TRY(check_view(&args->k, "k"));
-  FOX_TRY(check_view(&args->v, "v"));
-  FOX_TRY(check_view(&args->o, "o"));
-  FOX_TRY(check_extent(&args->k, args->dims.N, args->dims.D, "k"));
-  FOX_TRY(check_extent(&args->v, args->dims.N, args->dims.D, "v"));
-  if (!args->log_lambda || !args->lse) return fail(FOX_E_ARG, "log_lambda and lse must not be NULL");
-  fox::FwdK k{};
-  k.q = to_view(args->q);
-  k.k = to_view(args->k);
-  k.v = to_view(args->v);
-  k.o = to_view(args->o);
-  k.c = args->log_lambda;
-  k.lse = args->lse;
-  k.seq_start = args->seq_start;
-  k.thr = args->threshold;
-  k.first_block = args->first_block;
-  k.B = args->dims.B; k.H = args->dims.H; k.M = args->dims.M; k.N = args->dims.N;
-  k.sm_scale = args->sm_scale;
-  k.n_mtiles = (args->dims.M + fox::kFwdBM - 1) / fox::kFwdBM;
-  k.splits = 1;
-  if (args->workspace) {
-    int64_t need = 0;
-    FOX_TRY(fox_attn_fwd_workspace_bytes(&args->dims, &need));
-    if (need > 0) {
-      if (args->workspace_bytes < need) return fail(FOX_E_ARG, "workspace too small: %lld < %lld bytes", (long long)args->workspace_bytes, (long long)need);
-      if (((uintptr_t)args->workspace & 15) != 0) return fail(FOX_E_ALIGN, "workspace must be 16-byte aligned");
-      k.splits = fox::fwd_key_splits(k.B, k.H, k.M, k.N);
-      k.ws_o = (float*)args->workspace;
-      k.ws_ml = k.ws_o + (int64_t)k.splits * k.B * k.H * k.M * args->dims.D;
-    }
-  }
-  return check_hip(fox::launch_fwd(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), "fox_attn_fwd");
+  int64_t need = 0;
+  FOX_TRY(fox_attn_fwd_workspace_bytes(&args->dims, &need));
+  if (need > FOX_NOALLOC_SCRATCH_BYTES)
+    return fail(FOX_E_ARG, "fox_attn_fwd_noalloc: this shape needs %lld bytes of key-split scratch, the library holds %lld; "
+                "use fox_attn_fwd with a caller-provided workspace", (long long)need, (long long)FOX_NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (need > 0) FOX_TRY(scratch_of_current_device(&ws));
+  return fwd_impl(args, ws, need, stream, "fox_attn_fwd_noalloc");
 }
 
 int fox_attn_bwd_delta(const fox_bwd_args* args, void* stream) {

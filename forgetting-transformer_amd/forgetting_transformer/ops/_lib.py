@@ -113,6 +113,7 @@ SIGNATURES = {
     "fox_auto_threshold": (C.c_int, [C.POINTER(Dims), C.POINTER(View), C.POINTER(View), C.c_float, C.c_void_p, C.c_void_p,
                                      C.c_void_p]),
     "fox_attn_fwd": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),
+    "fox_attn_fwd_noalloc": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),
     "fox_attn_fwd_workspace_bytes": (C.c_int, [C.POINTER(Dims), C.POINTER(C.c_int64)]),
     "fox_attn_bwd_delta": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),
     "fox_attn_bwd_dkdv": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),

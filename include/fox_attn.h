@@ -129,6 +129,20 @@ int fox_attn_fwd(const fox_fwd_args* args, void* stream);
  */
 int fox_attn_fwd_workspace_bytes(const fox_dims* dims, int64_t* bytes);
 
+/*
+ * fox_attn_fwd for callers that cannot allocate device memory or bring a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same
+ * arguments and results as fox_attn_fwd (bit for bit), except that args->workspace / workspace_bytes are
+ * ignored: the partial results of a key-split forward go to a 64 MiB array that lives inside the library
+ * (one copy per GPU, held until the process ends).  The call allocates nothing.  A shape whose splits need
+ * more than 64 MiB (fox_attn_fwd_workspace_bytes) is rejected with FOX_E_ARG; shapes that are not split
+ * never touch the array.  The device that owns `stream` must be the current device.  All calls on one GPU
+ * share that GPU's array: calls that may overlap in time on one GPU (different streams, or graphs replayed
+ * concurrently) race on it; calls ordered on one stream do not.  Every element a call reads it has written
+ * before, so nothing needs clearing between calls.
+ */
+int fox_attn_fwd_noalloc(const fox_fwd_args* args, void* stream);
+
 typedef struct fox_bwd_args {
   fox_dims dims;
   fox_view q, k, v, o, d_o;   /* inputs */

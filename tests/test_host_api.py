@@ -277,3 +277,16 @@ def test_autograd_function_signature_matches_reference():
     sig = inspect.signature(forgetting_attention)
     assert [p for p in sig.parameters] == ["q", "k", "v", "log_fgate", "head_first", "seq_start", "sm_scale", "adaptive_threshold"]
     assert all(sig.parameters[p].kind is inspect.Parameter.KEYWORD_ONLY for p in ("head_first", "seq_start", "sm_scale", "adaptive_threshold"))
+
+
+def test_noalloc_rejects_shapes_beyond_its_array():
+    """The entry point that allocates nothing holds 64 MiB for key-split partials; a shape that needs more is refused
+    before anything touches the GPU."""
+    lib = _lib.load()
+    dims = _lib.Dims(7, 73, 128, 4096, 128, _lib.DTYPE_BF16)   # 511 query tiles x 2 splits: 68.0 MB > 64 MiB
+    need = C.c_int64(0)
+    _lib.check(lib.fox_attn_fwd_workspace_bytes(C.byref(dims), C.byref(need)), "fox_attn_fwd_workspace_bytes")
+    assert need.value > 64 << 20
+    args = _lib.FwdArgs(dims)
+    rc = lib.fox_attn_fwd_noalloc(C.byref(args), None)
+    assert rc == -1 and b"64" in lib.fox_last_error() and b"scratch" in lib.fox_last_error()
