@@ -41,7 +41,11 @@ int check_dims(const fox_dims* d) {
   if (d->M > d->N) return fail(FOX_E_ARG, "the key/value tensors must be at least as long as the query tensor (M=%d > N=%d)", d->M, d->N);
   if (d->D != 16 && d->D != 32 && d->D != 64 && d->D != 128) return fail(FOX_E_ARG, "head dim must be one of 16, 32, 64, 128 (got %d)", d->D);
   if (d->dtype != FOX_DTYPE_BF16 && d->dtype != FOX_DTYPE_FP16) return fail(FOX_E_ARG, "dtype must be FOX_DTYPE_BF16 or FOX_DTYPE_FP16 (got %d)", d->dtype);
-  if ((int64_t)d->B * d->H > 0x7fffffffLL / 4096) return fail(FOX_E_ARG, "B*H too large");
+  // B*H is the y extent of some grids (at most 65535), and every grid that folds (batch, head) into x
+  // must stay below 2^31 workgroups: tiles of at least 64 rows over the longer sequence.
+  if ((int64_t)d->B * d->H > 65535) return fail(FOX_E_ARG, "B*H must not exceed 65535 (got %lld)", (long long)d->B * d->H);
+  if ((int64_t)d->B * d->H * ((d->N + 63) / 64) * 64 > 0x7fffffffLL)
+    return fail(FOX_E_ARG, "B*H*ceil(N/64) must stay below 2^25 workgroups (got B*H = %lld, N = %d)", (long long)d->B * d->H, d->N);
   return FOX_OK;
 }
 

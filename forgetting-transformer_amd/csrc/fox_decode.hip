@@ -105,7 +105,6 @@ __global__ __launch_bounds__(256) void decode_kernel(const FwdK a) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) qf[e] *= qk_scale;
   }
-  const float cref2 = c_ref * kLog2e;
   float m = -3.0e38f, l = 0.f;  // finite floor: a group that has seen no key yet yields exp2(-inf) = 0
   float acc[8];
 #pragma unroll
@@ -135,8 +134,10 @@ __global__ __launch_bounds__(256) void decode_kernel(const FwdK a) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) dot = fmaf(qf[e], kf[e], dot);
       dot = row_sum<LPR>(dot);
-      // log2-domain score: sm_scale*log2e*(q.k) + (c_ref - c_n)*log2e
-      const float x = fmaf(-cn[u], kLog2e, dot + cref2);
+      // log2-domain score: sm_scale*log2e*(q.k) + (c_ref - c_n)*log2e.  The two cumulative sums are subtracted
+      // first (they are of similar, possibly large, magnitude; their difference is small and exact to an ulp of
+      // itself), then scaled: the order of the reference (:642-643).
+      const float x = fmaf(c_ref - cn[u], kLog2e, dot);
       s[u] = (base + u * KPL + r < k1) ? x : -INFINITY;
       bmax = fmaxf(bmax, s[u]);
     }

@@ -124,12 +124,14 @@ __device__ __forceinline__ void store_logit(void* p, int64_t i, float x) {
 
 // logsigmoid(x) = min(x, 0) - log1p(exp(-|x|)), stable on both sides, from the hardware exp / log:
 // log1p(z) for z in (0, 1] is log(u) + (z - (u - 1)) / u with u = fl(1 + z), which repairs the rounding
-// of 1 + z (absolute error ~1e-8, and log1p(z) -> z for tiny z as it must).
+// of 1 + z (absolute error ~1e-8, and log1p(z) -> z for tiny z as it must).  The result is clamped to <= 0:
+// a log gate is never positive, and the pruning bounds rely on the cumulative sums not increasing, whatever
+// the last bit of the hardware logarithm does near u = 1.
 __device__ __forceinline__ float log_sigmoid(float x) {
   const float z = __expf(-fabsf(x));
   const float u = 1.0f + z;
-  const float l = __logf(u) + __fdividef(z - (u - 1.0f), u);
-  return fminf(x, 0.f) - l;
+  const float l = fmaxf(__logf(u) + __fdividef(z - (u - 1.0f), u), 0.f);
+  return fminf(fminf(x, 0.f) - l, 0.f);
 }
 
 // c[n] = sum_{seq_start <= l <= n} logsigmoid(x[l]) in one pass over the logits; optionally also

@@ -8,11 +8,10 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from conftest import make_inputs
+from conftest import REL_TOL, make_inputs, rel_err
 from oracle import fox_oracle as O
 
 pytestmark = pytest.mark.gpu
-REL_TOL = 2e-2
 
 
 @pytest.fixture(scope="module")
@@ -22,11 +21,6 @@ def ops():
     from forgetting_transformer.ops import _lib
     _lib.load()
     return forgetting_attention, forgetting_attention_from_logits
-
-
-def rel_err(x, ref):
-    x, ref = x.float(), ref.float()
-    return (x - ref).abs().max().item() / max(1.0, ref.abs().max().item())
 
 
 @pytest.mark.parametrize("gate_dtype", [torch.bfloat16, torch.float16, torch.float32])
@@ -89,3 +83,29 @@ def test_fused_gate_with_pruning_and_extreme_logits(ops):
     assert torch.isfinite(xf.grad).all()
     assert rel_err(out_f, out_u) <= 1e-2
     assert rel_err(xf.grad, xu.grad) <= 1e-3
+
+
+@pytest.mark.parametrize("gate_dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_log_gates_are_never_positive_and_sums_never_increase(ops, gate_dtype):
+    """Extreme logits (around +-20 and +-80, zeros, the largest finite values of the dtype): logsigmoid from the
+    hardware exp / log must stay <= 0, so that the cumulative sums never increase -- the pruning-bound searches rely
+    on that order."""
+    import ctypes as C
+    from forgetting_transformer.ops import _lib
+    lib = _lib.load()
+    B, H, N = 2, 3, 6000
+    g = torch.Generator().manual_seed(5)
+    centres = torch.tensor([-80.0, -20.0, -1e-3, 0.0, 1e-3, 20.0, 80.0])
+    x = centres[torch.randint(0, 7, (B, H, N), generator=g)] + torch.randn(B, H, N, generator=g) * 0.5
+    x[0, 0, :4] = torch.tensor([float(torch.finfo(gate_dtype).max) if gate_dtype != torch.float32 else 3e38, 88.0, 16.7, 17.4])
+    x = x.to(gate_dtype).cuda()
+    log_fgate = torch.empty(B, H, N, device="cuda")
+    c = torch.empty(B, H, N, device="cuda")
+    dt = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16, torch.float32: _lib.DTYPE_FP32}[gate_dtype]
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.fox_gate_cumsum_fwd(x.data_ptr(), dt, *x.stride(), None, log_fgate.data_ptr(), c.data_ptr(), B, H, N, stream),
+               "fox_gate_cumsum_fwd")
+    assert torch.isfinite(log_fgate).all() and (log_fgate <= 0).all()
+    assert (c[..., 1:] <= c[..., :-1]).all()
+    want = F.logsigmoid(x.double())
+    assert (log_fgate.double() - want).abs().max().item() <= 1e-6 * max(1.0, want.abs().max().item())

@@ -5,7 +5,7 @@ the output (reference: model/forgetting_transformer/modeling_forgetting_transfor
 343-346, 366-423).  The projections themselves are plain matmuls and stay in torch on both sides.
 
 Forward and every gradient that flows back through the chain are compared with the operator's bar,
-max|x - ref| <= 2e-2 * max(1, max|ref|); the oracle chain runs in fp32 from the same 16-bit inputs.
+max|x - ref| <= 2e-2 * max|ref|; the oracle chain runs in fp32 from the same 16-bit inputs.
 """
 import math
 
@@ -13,10 +13,10 @@ import pytest
 import torch
 import torch.nn.functional as F
 
+from conftest import REL_TOL, rel_err
 from oracle import fox_oracle as O
 
 pytestmark = pytest.mark.gpu
-REL_TOL = 2e-2
 
 
 @pytest.fixture(scope="module")
@@ -26,11 +26,6 @@ def ft():
     from forgetting_transformer.ops import _lib
     _lib.load()
     return forgetting_transformer
-
-
-def rel_err(x, ref):
-    x, ref = x.float(), ref.float()
-    return (x - ref).abs().max().item() / max(1.0, ref.abs().max().item())
 
 
 def _leaves(B, T, H, D, seed):

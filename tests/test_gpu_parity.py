@@ -1,12 +1,12 @@
 """GPU parity tests: the HIP kernels, called through the C ABI by the Python
 operator, against the oracle on the same seeded inputs.
 
-Tolerance (bf16): max |x - ref| <= 2e-2 * max(1, max|ref|) for out, dq, dk, dv,
-dlog_fgate, the bound the benchmark configurations are judged by ("max-abs error 2e-2 relative to output scale",
-with the scale floored at 1 so that a reference that is zero up to rounding -- a row with
-a single valid key has dS = 0 exactly -- does not turn rounding noise into a relative error).  The
-reference's own grid (fp16) uses its own bound, atol = 1e-2
-(ops/forgetting_attention.py:1416-1425).
+Tolerance (bf16): max |x - ref| <= 2e-2 * max|ref| for out, dq, dk, dv, dlog_fgate, the bound the benchmark
+configurations are judged by ("max-abs error 2e-2 relative to output scale"; the scale is the reference's own
+maximum, without a floor, unless the reference is exactly zero everywhere -- a single valid key per row gives
+dS = 0 exactly), and row by row for out, dq, dk, dv: |x - ref| <= 2e-2 * max|ref row| + 6e-3 * max|ref|, so
+a wrong row of small magnitude cannot hide behind a large one.  The measured ratios are printed at the end of the run.  The reference's own grid
+(fp16) uses its own bound, atol = 1e-2 (ops/forgetting_attention.py:1416-1425).
 """
 import ctypes as C
 import math
@@ -16,12 +16,10 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from conftest import ROOT, make_inputs
+from conftest import REL_TOL, ROOT, assert_parity, make_inputs, rel_err
 from oracle import fox_oracle as O
 
 pytestmark = pytest.mark.gpu
-
-REL_TOL = 2e-2
 
 
 @pytest.fixture(scope="module")
@@ -31,12 +29,6 @@ def fa():
     from forgetting_transformer.ops import _lib
     _lib.load()  # fails loudly when the HIP library is missing
     return forgetting_attention
-
-
-def rel_err(x, ref):
-    x, ref = x.float(), ref.float()
-    scale = max(1.0, ref.abs().max().item())    # "2e-2 * max(1, scale of x_ref)"
-    return (x - ref).abs().max().item() / scale
 
 
 def run_case(fa, B, H, M, N, D, *, dtype=torch.bfloat16, head_first=True, thr=None, sm_scale=None, tol=REL_TOL,
@@ -54,8 +46,7 @@ def run_case(fa, B, H, M, N, D, *, dtype=torch.bfloat16, head_first=True, thr=No
             err = (x.float() - r.float()).abs().max().item()
             assert err <= atol, f"{name}: abs err {err:.3e} > {atol}"
         else:
-            e = rel_err(x, r)
-            assert e <= tol, f"{name}: rel err {e:.3e} > {tol}"
+            assert_parity(name, x, r, tol=tol, rows=name != "dlog_fgate")
     return got, ref, ss
 
 
@@ -72,7 +63,7 @@ def test_golden_forward_backward(fa):
     out = fa(q, k, v, g, head_first=True, seq_start=ss, sm_scale=0.25)
     out.backward(do)
     for name, x in (("out", out), ("dq", q.grad), ("dk", k.grad), ("dv", v.grad), ("dlog_fgate", g.grad)):
-        assert rel_err(x, torch.from_numpy(d[name]).cuda()) <= REL_TOL, name
+        assert_parity(name, x, torch.from_numpy(d[name]).cuda(), rows=name != "dlog_fgate")
     # batch row 1 starts at key 150 = query 22: queries 0..21 attend to nothing
     assert (out[1, :, :22] == 0).all() and (q.grad[1, :, :22] == 0).all()
     assert (k.grad[1, :, :150] == 0).all() and (v.grad[1, :, :150] == 0).all()
@@ -225,8 +216,8 @@ def test_fox_layer_views(fa):
     assert out.stride() == q.stride()                 # the un-permute on return stays free
     out.backward(do)
     ref = O.forgetting_attention_ref_grads(q.detach(), k.detach(), v.detach(), gates.detach(), do, head_first=True, seq_start=ss)
-    for x_, r in zip((out, q.grad, k.grad, v.grad, gates.grad), ref):
-        assert rel_err(x_, r) <= REL_TOL
+    for name, x_, r in zip(("out", "dq", "dk", "dv", "dlog_fgate"), (out, q.grad, k.grad, v.grad, gates.grad), ref):
+        assert_parity(name, x_, r, rows=name != "dlog_fgate")
 
 
 @pytest.mark.parametrize("Z,H,M,N,D", [(4, 2, 1020, 2098, 64), (4, 2, 1024, 2048, 128)])
@@ -426,8 +417,9 @@ def test_random_configurations(fa, case):
         worst = float(thr) if thr_kind == "float" else float(thr.max().item())
         tol = tol + 4.0 * N * math.exp(worst)    # mass a row can lose: at most N entries of weight e^thr (scores are O(1))
     for name, x, r in zip(("out", "dq", "dk", "dv", "dlog_fgate"), (out, q.grad, k.grad, v.grad, g.grad), ref):
-        assert torch.isfinite(x).all(), (name, case)
-        assert rel_err(x, r) <= tol, (name, case, rel_err(x, r), tol, dict(B=B, H=H, M=M, N=N, D=D, thr=thr_kind))
+        # floor: shapes with one or two keys have gradients that vanish by cancellation (inputs are O(1))
+        assert_parity(name, x, r, tol=tol, rows=name != "dlog_fgate", floor=0.05,
+                      context=(case, dict(B=B, H=H, M=M, N=N, D=D, thr=thr_kind)))
 
 
 @pytest.mark.parametrize("D", [16, 32, 64])
@@ -443,55 +435,96 @@ def test_long_sequences_at_small_head_dims(fa, D, M, N, seq, thr):
     out.backward(do)
     tol = REL_TOL + (4.0 * N * math.exp(thr) if thr is not None else 0.0)
     for name, x, r in zip(("out", "dq", "dk", "dv", "dlog_fgate"), (out, q.grad, k.grad, v.grad, g.grad), ref):
-        assert torch.isfinite(x).all(), name
-        assert rel_err(x, r) <= tol, (name, rel_err(x, r), tol)
+        assert_parity(name, x, r, tol=tol, rows=name != "dlog_fgate")
 
 
 # --------------------------------------------------------------------------------------
 # benchmark configurations 3-5 at full size
 # --------------------------------------------------------------------------------------
-def _full_size_check(fa, B, H, T, D, mean, std, thr, pairs):
+# One (batch, head) pair per XCD: the workgroup -> (batch, head) map of the kernels puts pair bh on XCD bh mod 8,
+# and with H = 16 that is h mod 8.
+ALL_XCD_PAIRS = [(0, 0), (0, 9), (1, 2), (1, 11), (2, 4), (2, 13), (3, 6), (3, 15)]
+
+
+def _full_size_check(fa, B, H, T, D, mean, std, thr, pairs, seq_start=None):
     g_ = torch.Generator(device="cuda").manual_seed(3)
     q, k, v = (torch.randn(B, T, H, D, generator=g_, device="cuda").bfloat16().requires_grad_() for _ in range(3))
     gates = F.logsigmoid(torch.randn(B, T, H, generator=g_, device="cuda") * std + mean).requires_grad_()
     do = torch.randn(B, T, H, D, generator=g_, device="cuda").bfloat16()
-    out = fa(q, k, v, gates, adaptive_threshold=thr)
+    ss = None if seq_start is None else torch.tensor(seq_start, device="cuda")
+    out = fa(q, k, v, gates, adaptive_threshold=thr, seq_start=ss)
     out.backward(do)
     got = (out, q.grad, k.grad, v.grad)
     for x in got + (gates.grad,):
         assert torch.isfinite(x).all()
-    # property: the gate gradient of position 0 is sum_n dc_n = 0
-    assert gates.grad[:, 0].abs().max() <= 1e-3 * max(1.0, gates.grad.abs().max().item())
-    for b, h in pairs:   # oracle on a few (batch, head) pairs: one pair needs a 1 GiB score matrix
+    # property: the gate gradient of every position up to seq_start (position 0 without padding) is sum_n dc_n = 0
+    for b in range(B):
+        upto = 1 if ss is None else int(ss[b]) + 1
+        assert gates.grad[b, :upto].abs().max() <= 1e-3 * gates.grad.abs().max().item(), b
+    for b, h in pairs:   # oracle on (batch, head) pairs: one pair needs a 1 GiB score matrix
         sl = lambda x: x.detach()[b:b + 1, :, h:h + 1]
-        ref = O.forgetting_attention_ref_grads(sl(q), sl(k), sl(v), gates.detach()[b:b + 1, :, h:h + 1], sl(do))
+        ref = O.forgetting_attention_ref_grads(sl(q), sl(k), sl(v), gates.detach()[b:b + 1, :, h:h + 1], sl(do),
+                                               seq_start=None if ss is None else ss[b:b + 1])
         for name, x, r in zip(("out", "dq", "dk", "dv"), got, ref):
-            assert rel_err(sl(x), r) <= REL_TOL, (name, b, h)
-        assert rel_err(gates.grad[b:b + 1, :, h:h + 1], ref[4]) <= REL_TOL, ("dlog_fgate", b, h)
+            assert_parity(name, sl(x), r, context=(b, h))
+        assert_parity("dlog_fgate", gates.grad[b:b + 1, :, h:h + 1], ref[4], rows=False, context=(b, h))
     return out.detach()
 
 
 def test_config3_long_context(fa):
-    _full_size_check(fa, 4, 16, 16384, 128, 3.0, 1.0, None, [(0, 0), (3, 15)])
+    _full_size_check(fa, 4, 16, 16384, 128, 3.0, 1.0, None, ALL_XCD_PAIRS)
+
+
+def test_config3_shape_with_left_padding(fa):
+    """The long-context shape with left padding, forward and backward: padding inside the first tile, across many
+    tiles, ending mid-tile just below the middle, and leaving only the last 300 positions."""
+    _full_size_check(fa, 4, 16, 16384, 128, 3.0, 1.0, None, ALL_XCD_PAIRS, seq_start=[5, 3000, 8191, 16084])
 
 
 def test_config4_pruned(fa):
-    base = _full_size_check(fa, 4, 16, 16384, 128, -1.0, 2.0, None, [(1, 7)])
+    base = _full_size_check(fa, 4, 16, 16384, 128, -1.0, 2.0, None, ALL_XCD_PAIRS)
     for thr in ("auto", -10.0):
-        out = _full_size_check(fa, 4, 16, 16384, 128, -1.0, 2.0, thr, [(1, 7)])
+        out = _full_size_check(fa, 4, 16, 16384, 128, -1.0, 2.0, thr, ALL_XCD_PAIRS)
         assert rel_err(out, base) <= 1e-3     # pruned mass <= e^-10: far below bf16 rounding
+
+
+def _cache_inputs(B, H, M, N, D, mean, std, seed):
+    g_ = torch.Generator(device="cuda").manual_seed(seed)
+    q = torch.randn(B, H, M, D, generator=g_, device="cuda").bfloat16()
+    k = torch.randn(B, H, N, D, generator=g_, device="cuda").bfloat16()
+    v = torch.randn(B, H, N, D, generator=g_, device="cuda").bfloat16()
+    gates = F.logsigmoid(torch.randn(B, H, N, generator=g_, device="cuda") * std + mean)
+    ss = torch.randint(0, 8192, (B,), generator=g_, device="cuda")
+    return q, k, v, gates, ss
 
 
 @pytest.mark.parametrize("M", [128, 1])
 def test_config5_chunked_prefill_and_decode(fa, M):
     B, H, N, D = 16, 16, 32768, 128
-    g_ = torch.Generator(device="cuda").manual_seed(5)
-    q = torch.randn(B, H, M, D, generator=g_, device="cuda").bfloat16()
-    k = torch.randn(B, H, N, D, generator=g_, device="cuda").bfloat16()
-    v = torch.randn(B, H, N, D, generator=g_, device="cuda").bfloat16()
-    gates = F.logsigmoid(torch.randn(B, H, N, generator=g_, device="cuda") + 2.0)
-    ss = torch.randint(0, 8192, (B,), generator=g_, device="cuda")
+    q, k, v, gates, ss = _cache_inputs(B, H, M, N, D, 2.0, 1.0, 5)
     out = fa(q, k, v, gates, head_first=True, seq_start=ss)
     for b in range(B):
         ref = O.forgetting_attention_ref(q[b:b + 1], k[b:b + 1], v[b:b + 1], gates[b:b + 1], head_first=True, seq_start=ss[b:b + 1])
-        assert rel_err(out[b:b + 1], ref) <= REL_TOL, b
+        assert_parity("out", out[b:b + 1], ref, context=b)
+
+
+@pytest.mark.parametrize("M", [128, 1])
+@pytest.mark.parametrize("thr", [None, "auto"])
+def test_cache_shapes_under_strong_decay(fa, M, thr):
+    """The chunked-prefill (key-split tiled kernel) and decode (streaming kernel) shapes with the strongly decaying
+    gates of the pruned configuration, logits ~ N(-1, 2): the cumulative sums reach ~ -7e4 at N = 32768 (fp32 ulp
+    2^-7), so a kernel that rounds a score at the magnitude of the cumulative sums instead of forming the difference
+    of two nearby sums first loses the result.  out and the log-normaliser, every batch, against the oracle."""
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    B, H, N, D = 16, 16, 32768, 128
+    q, k, v, gates, ss = _cache_inputs(B, H, M, N, D, -1.0, 2.0, 6)
+    ss = (ss * 4 - 1000).clamp_min(0)   # up to 31764: some batches keep only the last few hundred keys
+    out, lse, _ = ForgettingAttention.apply(q, k, v, gates, ss, True, None, thr, True, False)
+    assert torch.cumsum(gates[0, 0], 0)[-1].item() < -2e4
+    for b in range(B):
+        # fp64 oracle: its cumulative sums are exact where an fp32 running sum of 32768 terms is not; the operator's
+        # own sums are correctly rounded fp32 (half an ulp, 4e-3 at 7e4), which bounds the error of a score and of lse
+        ref, lse_ref = O.forgetting_attention_ref(q[b:b + 1], k[b:b + 1], v[b:b + 1], gates[b:b + 1], head_first=True,
+                                                  seq_start=ss[b:b + 1], return_lse=True, compute_dtype=torch.float64)
+        assert_parity("out", out[b:b + 1], ref, context=b)
+        assert torch.isfinite(lse[b]).all() and (lse[b].double() - lse_ref[0]).abs().max().item() <= 2e-2, b

@@ -10,6 +10,7 @@ import math
 import pytest
 import torch
 
+from conftest import REL_TOL, rel_err
 from oracle import fox_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -22,11 +23,6 @@ def ft():
     from forgetting_transformer.ops import _lib
     _lib.load()
     return forgetting_transformer
-
-
-def rel_err(x, ref):
-    """max |x - ref| over max(1, scale of ref): the measure of the attention parity tests (bar 2e-2)."""
-    return (x.float() - ref.float()).abs().max().item() / max(1.0, ref.float().abs().max().item())
 
 
 def _close(got, want_fp32, dtype, ulps=2.0):
