@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+from collections import defaultdict
 from typing import Literal, Optional, Union
 
 import torch
@@ -52,22 +53,65 @@ def _stream(device: torch.device):
 class ForgettingAttention(torch.autograd.Function):
     """Autograd node; argument list identical to the reference's (``:72-73``).
 
-    ``record_time_key`` / ``record_attention_time`` / ``record_find_index_time``
-    (the reference's in-op CUDA-event timers, ``:45-70``) are accepted for
-    signature compatibility but must be off: kernels here are timed from outside
-    with a profiler.
+    ``record_time_key`` / ``record_attention_time`` / ``record_find_index_time`` are the
+    reference's in-op timers (``:45-70, 176-181, 217-222, 301-306, 358-363, 394-399``):
+    with ``record_attention_time`` the forward and the backward are bracketed by events on
+    the current stream, the host waits for the end event (as the reference synchronises)
+    and the milliseconds are added to ``ForgettingAttention.info[record_time_key]``
+    (``fwd_time`` / ``fwd_count`` / ``bwd_time`` / ``bwd_count``).  The pruning bounds are
+    searched inside the attention kernels here, not by kernels of their own, so
+    ``record_find_index_time`` only counts calls (``*_find_index_count``); the
+    ``*_find_index_time`` entries stay 0.0.
     """
+
+    info = defaultdict(lambda: {
+        "fwd_time": 0.0, "fwd_count": 0, "bwd_time": 0.0, "bwd_count": 0,
+        "fwd_find_index_time": 0.0, "fwd_find_index_count": 0,
+        "bwd_find_index_kv_time": 0.0, "bwd_find_index_kv_count": 0,
+        "bwd_find_index_q_time": 0.0, "bwd_find_index_q_count": 0,
+    })
+    events = defaultdict(lambda: {name: torch.cuda.Event(enable_timing=True)
+                                  for name in ("fwd_start_event", "fwd_end_event", "bwd_start_event", "bwd_end_event")})
 
     @staticmethod
     def forward(ctx, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
                 return_log_normalizer=False, return_start_index=False, record_time_key=None,
                 record_attention_time=False, record_find_index_time=False):
-        return _forward(ctx, False, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
-                        return_log_normalizer, return_start_index, record_attention_time, record_find_index_time)
+        cls = ForgettingAttention
+        if record_attention_time:
+            cls.events[record_time_key]["fwd_start_event"].record()
+        outs = _forward(ctx, False, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
+                        return_log_normalizer, return_start_index)
+        ctx.record_time_key = record_time_key
+        ctx.record_attention_time = record_attention_time
+        ctx.record_find_index_time = record_find_index_time
+        if record_find_index_time and adaptive_threshold is not None:
+            cls.info[record_time_key]["fwd_find_index_count"] += 1
+        if record_attention_time:
+            ev = cls.events[record_time_key]
+            ev["fwd_end_event"].record()
+            ev["fwd_end_event"].synchronize()
+            cls.info[record_time_key]["fwd_time"] += ev["fwd_start_event"].elapsed_time(ev["fwd_end_event"])
+            cls.info[record_time_key]["fwd_count"] += 1
+        return outs
 
     @staticmethod
     def backward(ctx, do, *ignored):
-        return _backward(ctx, do) + (None,) * 9
+        cls = ForgettingAttention
+        key = ctx.record_time_key
+        if ctx.record_attention_time:
+            cls.events[key]["bwd_start_event"].record()
+        grads = _backward(ctx, do)
+        if ctx.record_find_index_time and ctx.saved_tensors[7] is not None:
+            cls.info[key]["bwd_find_index_kv_count"] += 1
+            cls.info[key]["bwd_find_index_q_count"] += 1
+        if ctx.record_attention_time:
+            ev = cls.events[key]
+            ev["bwd_end_event"].record()
+            ev["bwd_end_event"].synchronize()
+            cls.info[key]["bwd_time"] += ev["bwd_start_event"].elapsed_time(ev["bwd_end_event"])
+            cls.info[key]["bwd_count"] += 1
+        return grads + (None,) * 9
 
 
 class ForgettingAttentionFromLogits(torch.autograd.Function):
@@ -80,7 +124,7 @@ class ForgettingAttentionFromLogits(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, fgate_logit, seq_start, sm_scale, adaptive_threshold):
         out = _forward(ctx, True, q, k, v, fgate_logit, seq_start, True, sm_scale, adaptive_threshold,
-                       False, False, False, False)
+                       False, False)
         ctx.mark_non_differentiable(ctx.log_fgate)
         return out, ctx.log_fgate
 
@@ -93,10 +137,8 @@ _GATE_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16,
 
 
 def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
-             return_log_normalizer, return_start_index, record_attention_time, record_find_index_time):
+             return_log_normalizer, return_start_index):
     assert causal, "Only causal attention is supported"
-    assert not (record_attention_time or record_find_index_time), \
-        "in-op timers are not implemented; profile the kernels with rocprofv3 instead"
     Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
     assert Dq == Dk == Dv, "feature size of q, k, v should be equal"
     assert Dk in {16, 32, 64, 128}, "We only support head dims in {16, 32, 64, 128}"

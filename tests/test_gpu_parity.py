@@ -253,6 +253,28 @@ def test_log_normalizer_and_start_index_outputs(fa):
     assert si.dtype == torch.long and si.shape == (2, 3, 3)
 
 
+def test_in_op_timers_fill_the_info_table(fa):
+    """The reference's hidden timing flags (:45-70, :176-181, :217-222): same results, and the class-level table
+    gets the elapsed milliseconds and call counts under the caller's key."""
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    q, k, v, g, do, _ = make_inputs(2, 2, 512, 512, 64, device="cuda", seed=31, requires_grad=True)
+    plain = fa(q, k, v, g, head_first=True, adaptive_threshold=-20.0)
+    plain.backward(do)
+    want = [t.clone() for t in (plain, q.grad, k.grad, v.grad, g.grad)]
+    q.grad = k.grad = v.grad = g.grad = None
+    key = "timed-layer"
+    ForgettingAttention.info.pop(key, None)
+    for _ in range(2):
+        out = ForgettingAttention.apply(q, k, v, g, None, True, None, -20.0, False, False, key, True, True)
+        out.backward(do)
+    info = ForgettingAttention.info[key]
+    assert info["fwd_count"] == 2 and info["bwd_count"] == 2 and info["fwd_time"] > 0 and info["bwd_time"] > 0
+    assert info["fwd_find_index_count"] == 2 and info["bwd_find_index_kv_count"] == 2 and info["bwd_find_index_q_count"] == 2
+    assert torch.equal(out, want[0])
+    for got, w in zip((q.grad, k.grad, v.grad, g.grad), want[1:]):
+        assert torch.equal(got, 2 * w)       # two backward passes accumulated
+
+
 def test_pruning_bounds_match_the_scan_bit_exactly(fa):
     """first_block from the kernel's wave-parallel search == the reference's two-pointer scan
     (restated in C) run on the kernel's own cumulative sums."""
