@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the Forgetting Attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode|shift|norm_gate] [--no-extras] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode|c3d64|c3d32|c3d16|shift|norm_gate|ref_sweep]
+                    [--no-extras] [--no-cpu-baseline]
 
 A step is one forward + backward pass of ``forgetting_attention`` over one batch
 of synthetic input already resident in HBM (forward only for c5).  The default
@@ -17,7 +18,11 @@ Besides the headline value the line carries
                  attention, forward only, on this host's cores, bounded to ~10 s;
   acp          : pruned-tile fraction and speed-up of Adaptive Computation Pruning
                  (thresholds "auto" and -10.0) on strongly decaying gates;
-  prefill      : chunked-prefill shape (M=128, N=32768, left padding), HBM GB/s.
+  prefill      : chunked-prefill shape (M=128, N=32768, left padding), HBM GB/s;
+  decode       : one new token against the same cache;
+  head_dim_*   : the headline step at head dims 64, 32 and 16 (same token count and matmul work);
+  library_example : the small B4 T512 H12 D64 step, wall time against the sum of its kernels.
+--workload ref_sweep runs the reference's own benchmark recipe (its __main__ block) instead.
 """
 from __future__ import annotations
 
@@ -39,15 +44,47 @@ import torch  # noqa: E402
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0
 
-# HBM bytes per launch of the dominant kernel of a workload (fetched + written), from two rocprofv3 --pmc
-# passes over this script (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for the
-# plain 1 GiB copies of --copy-calibration (fetch x2.00, write x1.00); profiles/hbm_traffic_c3_c5.md.
-# Counters cannot be read from inside the timed run, so the figure is carried here.
-MEASURED_TRAFFIC_BYTES = {"c3": (2.049 + 0.504) * 2**30, "c5": (3.442 + 0.032) * 2**30, "decode": (3.565 + 0.001) * 2**30}
+# HBM bytes per launch of the dominant kernel of a workload (fetched + written) come from two rocprofv3 --pmc
+# passes over this script (FETCH_SIZE, WRITE_SIZE; counters cannot be read from inside the timed run).  The
+# summary of those passes, profiles/hbm_traffic_c3_c5.md, ends with a machine-readable block: the bytes per
+# workload and the SHA-256 of the kernel sources they were measured on.  measured_traffic() returns the figure
+# only while those sources are unchanged; otherwise the roofline carries traffic = null and says why.
+TRAFFIC_PROFILE = ROOT / "profiles" / "hbm_traffic_c3_c5.md"
+KERNEL_SOURCES = ["fox_common.hpp", "fox_kernels.hpp", "fox_fwd.hip", "fox_bwd.hip", "fox_decode.hip"]
+
+
+def kernel_source_digest():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        h.update((ROOT / "forgetting-transformer_amd" / "csrc" / name).read_bytes())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    """(bytes per launch or None, provenance string)."""
+    import re
+    if not TRAFFIC_PROFILE.exists():
+        return None, "no HBM traffic profile committed"
+    m = re.search(r"```json traffic\n(.*?)\n```", TRAFFIC_PROFILE.read_text(), flags=re.S)
+    if not m:
+        return None, f"{TRAFFIC_PROFILE.name} has no traffic block"
+    block = json.loads(m.group(1))
+    rel = f"profiles/{TRAFFIC_PROFILE.name}"
+    if workload not in block["bytes_per_launch"]:
+        return None, f"{rel} has no entry for {workload}"
+    if block["kernel_source_digest"] != kernel_source_digest():
+        return None, (f"{rel} was measured on kernel sources {block['kernel_source_digest']}, the tree holds "
+                      f"{kernel_source_digest()}: re-run its two rocprofv3 --pmc passes")
+    return float(block["bytes_per_launch"][workload]), f"{rel} (kernel sources {block['kernel_source_digest']})"
+
 
 WORKLOADS = {
     # name: B, T(M), N, H, D, gate mean, gate std, head_first, fwd_only, seq_start
     "c2": dict(B=4, M=512, N=512, H=12, D=64, mean=0.0, std=1.0, head_first=False, fwd_only=False, pad=False),
+    # config 3 at the other head dims: same token count and matmul work, the heads scaled up
+    "c3d32": dict(B=4, M=16384, N=16384, H=64, D=32, mean=3.0, std=1.0, head_first=False, fwd_only=False, pad=False),
+    "c3d16": dict(B=4, M=16384, N=16384, H=128, D=16, mean=3.0, std=1.0, head_first=False, fwd_only=False, pad=False),
     "c3": dict(B=4, M=16384, N=16384, H=16, D=128, mean=3.0, std=1.0, head_first=False, fwd_only=False, pad=False),
     # config 3 at the head dim of the reference's own models (hidden_size / num_heads = 64 in every
     # configs/experiment/longcrawl64/forgetting_transformer/*.yaml): same token count and matmul work, twice the heads
@@ -164,15 +201,14 @@ def stage_times(w, tensors, iters, threshold=None):
     out["fwd"] = event_time(f, iters)
     if w["fwd_only"]:
         return out
-    delta = torch.empty_like(lse)
+    delta = torch.empty((2,) + tuple(lse.shape), dtype=torch.float32, device=dev)
     dc = torch.empty_like(c)
     dg = torch.empty_like(c)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     bwd = _lib.BwdArgs(dims, _view(q), _view(k), _view(v), _view(o), _view(dout), _view(dq), _view(dk), _view(dv),
                        c.data_ptr(), lse.data_ptr(), ss, thr, 1.0 / math.sqrt(D), delta.data_ptr(), dc.data_ptr(),
                        dg.data_ptr())
-    for name, fn in (("bwd_delta", lib.fox_attn_bwd_delta), ("bwd_dkdv", lib.fox_attn_bwd_dkdv),
-                     ("bwd_dq", lib.fox_attn_bwd_dq)):
+    for name, fn in (("bwd_dq", lib.fox_attn_bwd_dq), ("bwd_dkdv", lib.fox_attn_bwd_dkdv)):
         out[name] = event_time(lambda fn=fn, name=name: _lib.check(fn(C.byref(bwd), stream), name), iters)
     out["cumsum_bwd"] = event_time(
         lambda: _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg.data_ptr(), B, H, N, stream), "cumsum_bwd"), iters)
@@ -276,7 +312,7 @@ def acp_report(steps, warmup):
     q, k, v, log_fgate = (x.detach() for x in (q, k, v, log_fgate))
     st = stage_times(w, (q, k, v, log_fgate, dout, None), max(3, steps), threshold=-10.0)
     S, R = w["B"] * w["H"] * w["M"] * w["D"] * 2, w["B"] * w["H"] * w["M"] * 4
-    alg = {"fwd": 4 * S + 2 * R, "bwd_delta": 2 * S + R, "bwd_dkdv": 6 * S + 4 * R, "bwd_dq": 5 * S + 4 * R}
+    alg = {"fwd": 4 * S + 2 * R, "bwd_dq": 6 * S + 5 * R, "bwd_dkdv": 6 * S + 6 * R}
     rep["pruned_kernels"] = {k_: {"ms": st[k_] * 1e3, "algorithmic_gbps": alg[k_] / st[k_] * 1e-9} for k_ in alg}
     return rep
 
@@ -326,13 +362,13 @@ def decode_report(steps, warmup):
             "kernel_hbm_gbps": alg / st["fwd"] * 1e-9, "kernel_frac_of_8TBps": alg / st["fwd"] * 1e-9 / PEAK_HBM_GBPS}
 
 
-def head_dim_report(steps, warmup):
-    """The headline step at head dim 64 (what every model configuration of the reference uses:
-    configs/experiment/longcrawl64/forgetting_transformer/*.yaml have hidden_size / num_heads = 64),
-    same token count and matmul work as the D = 128 workload."""
+def head_dim_report(steps, warmup, name="c3d64"):
+    """The headline step at another head dim, same token count and matmul work as the D = 128 workload: 64 (what
+    every model configuration of the reference uses: configs/experiment/longcrawl64/forgetting_transformer/*.yaml
+    have hidden_size / num_heads = 64), 32 and 16 (the remaining tile specialisations)."""
     from forgetting_transformer import forgetting_attention
 
-    w = WORKLOADS["c3d64"]
+    w = WORKLOADS[name]
     tensors = synth(w, "cuda")
     q, k, v, log_fgate, dout, _ = tensors
     q, k, v, log_fgate = (x.requires_grad_() for x in (q, k, v, log_fgate))
@@ -348,6 +384,97 @@ def head_dim_report(steps, warmup):
            "kernels": {name: {"ms": st[name] * 1e3, "tflops": m * unit / st[name] * 1e-12}
                        for name, m in (("fwd", 2), ("bwd_dkdv", 4), ("bwd_dq", 3))}}
     return rep
+
+
+def small_shape_report(steps, warmup):
+    """The library-example shape (B4 T512 H12 D64 bf16 fwd+bwd): launch-latency-bound.  Wall time per step of the
+    operator (Python, autograd, allocations, launches), the same step replayed from a HIP graph, and the sum of
+    its kernels timed alone."""
+    from forgetting_transformer import forgetting_attention
+
+    w = WORKLOADS["c2"]
+    tensors = synth(w, "cuda", seed=2)
+    q, k, v, log_fgate, dout, _ = tensors
+    q, k, v, log_fgate = (x.requires_grad_() for x in (q, k, v, log_fgate))
+
+    def step():
+        forgetting_attention(q, k, v, log_fgate).backward(dout)
+        q.grad = k.grad = v.grad = log_fgate.grad = None
+    t = time_steps(step, max(steps, 50), max(warmup, 5))
+    t_graph = graph_time(step, max(steps, 50))
+    st = stage_times(w, tensors, max(steps, 20))
+    path = ("cumsum_fwd", "fwd", "bwd_dq", "bwd_dkdv", "cumsum_bwd")
+    return {"workload": "B4 T512 H12 D64 bf16 fwd+bwd, gate logits N(0,1)", "wall_ms_per_step": t * 1e3,
+            "graph_replay_ms_per_step": t_graph * 1e3, "kernel_sum_ms": sum(st[n] for n in path) * 1e3,
+            "kernels_ms": {n: st[n] * 1e3 for n in path}}
+
+
+def ref_sweep_report(ns):
+    """The reference's own benchmark recipe (ops/forgetting_attention.py:1438-1513): B4 H32 D64 bf16, head-first,
+    N_CTX = 2^10 .. 2^14, gate logits ~ U(0,10), sm_scale = 1.3, threshold -10 per (batch, head); forward and
+    backward (o.backward(do, retain_graph=True), gradients accumulating) timed separately like
+    triton.testing.do_bench: events around every call, the cache flushed by zeroing a buffer before each, about
+    25 ms of warm-up and 100 ms of timed calls, mean.  FLOPs as there: forward 2*B*H*N^2*D (causal), backward
+    2.5 x forward.  One JSON line."""
+    from forgetting_transformer import forgetting_attention
+
+    B, H, D = 4, 32, 64
+    dev = "cuda"
+    flush = torch.empty(512 << 20, dtype=torch.int8, device=dev)   # larger than the 256 MiB last-level cache
+
+    def do_bench(fn, warmup_ms=25.0, rep_ms=100.0):
+        fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(5):
+            flush.zero_()
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        est = s.elapsed_time(e) / 5
+        n_warm, n_rep = max(1, int(warmup_ms / est)), max(3, int(rep_ms / est))
+        for _ in range(n_warm):
+            fn()
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(n_rep)]
+        ends = [torch.cuda.Event(enable_timing=True) for _ in range(n_rep)]
+        for i in range(n_rep):
+            flush.zero_()
+            starts[i].record()
+            fn()
+            ends[i].record()
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in zip(starts, ends)) / n_rep
+
+    rows = []
+    for n_ctx in [2 ** i for i in range(10, 15)]:
+        g = torch.Generator(device=dev).manual_seed(n_ctx)
+        q, k, v = (torch.randn((B, H, n_ctx, D), generator=g, device=dev, dtype=torch.float32).bfloat16().requires_grad_()
+                   for _ in range(3))
+        logit = torch.empty((B, H, n_ctx), dtype=torch.float32, device=dev).uniform_(0, 10, generator=g)
+        log_fgate = torch.nn.functional.logsigmoid(logit).requires_grad_()
+        thr = torch.full((B, H), -10.0, dtype=torch.float, device=dev)
+        fwd = lambda: forgetting_attention(q, k, v, log_fgate, head_first=True, sm_scale=1.3, adaptive_threshold=thr)
+        ms_f = do_bench(fwd)
+        o = fwd()
+        do = torch.randn(o.shape, generator=g, device=dev, dtype=torch.float32).bfloat16()
+        ms_b = do_bench(lambda: o.backward(do, retain_graph=True))
+        f_fwd = 2.0 * B * H * n_ctx * n_ctx * D     # 2 matmuls x 2*B*H*N^2*D, halved for the causal mask
+        rows.append({"N_CTX": n_ctx, "fwd_ms": ms_f, "fwd_tflops": f_fwd / ms_f * 1e-9, "bwd_ms": ms_b,
+                     "bwd_tflops": 2.5 * f_fwd / ms_b * 1e-9})
+        del q, k, v, log_fgate, o, do
+    top = rows[-1]
+    total_ms = top["fwd_ms"] + top["bwd_ms"]
+    value = 3.5 * 2.0 * B * H * top["N_CTX"] ** 2 * D / total_ms * 1e-9
+    print(json.dumps({
+        "metric": "reference benchmark recipe: fwd and bwd TFLOP/s over N_CTX (value: fwd+bwd at N_CTX=16384)",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": ns.steps, "warmup": ns.warmup, "ms_per_step": total_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "ref_sweep: B4 H32 D64 bf16 head_first, N_CTX 1024..16384, gate logits U(0,10), sm_scale 1.3, "
+                               "adaptive_threshold -10 per (batch, head); ops/forgetting_attention.py:1438-1513",
+                   "flops_convention": "fwd 2*B*H*N^2*D, bwd 2.5 x fwd (causal)", "timing": "events per call, cache flushed before "
+                   "each call, ~25 ms warm-up, ~100 ms timed, mean (triton.testing.do_bench)"},
+        "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS, "sweep": rows}))
 
 
 def shift_report(ns):
@@ -391,7 +518,7 @@ def shift_report(ns):
         "config": {"workload": f"shift: B{B} T{T} H{H} D{D} bf16 fwd+bwd, weights fp32 (B,T,H)"},
         "roofline": {"kernel": "shift_bwd", "bound": "hbm", "achieved": kernels["shift_bwd"]["gbps"], "peak": PEAK_HBM_GBPS,
                      "unit": "GB/s", "frac": kernels["shift_bwd"]["gbps"] / PEAK_HBM_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get("shift"), "algorithmic_bytes": bytes_b,
+                     "traffic": None, "algorithmic_bytes": bytes_b,
                      "avg_launch_ms": t_b * 1e3},
         "kernels": kernels,
     }
@@ -451,7 +578,7 @@ def norm_gate_report(ns):
         "config": {"workload": f"norm_gate: B{B} T{T} heads{G} D{D} bf16 fwd+bwd, sigmoid gate, fp32 weight"},
         "roofline": {"kernel": "norm_gate_bwd", "bound": "hbm", "achieved": kernels["norm_gate_bwd"]["gbps"],
                      "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": kernels["norm_gate_bwd"]["gbps"] / PEAK_HBM_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get("norm_gate"), "algorithmic_bytes": bytes_b,
+                     "traffic": None, "algorithmic_bytes": bytes_b,
                      "avg_launch_ms": t_b * 1e3},
         "kernels": kernels,
     }
@@ -463,7 +590,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift", "norm_gate"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift", "norm_gate", "ref_sweep"])
     ap.add_argument("--no-extras", action="store_true", help="skip the ACP and chunked-prefill reports")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -489,6 +616,8 @@ def main():
         return shift_report(ns)
     if ns.workload == "norm_gate":
         return norm_gate_report(ns)
+    if ns.workload == "ref_sweep":
+        return ref_sweep_report(ns)
 
     w = WORKLOADS[ns.workload]
     tensors = synth(w, "cuda")
@@ -520,7 +649,7 @@ def main():
             e["tflops"] = kern_flops[name] / t * 1e-12
             e["frac_of_peak"] = e["tflops"] / PEAK_BF16_TFLOPS
         kernels[name] = e
-    traffic = MEASURED_TRAFFIC_BYTES.get(ns.workload)
+    traffic, traffic_source = measured_traffic(ns.workload)
     if w["fwd_only"]:  # few query rows against a long key sequence: one pass over K and V, HBM-bound
         dom = "fwd"
         pad = seq_start.float() if seq_start is not None else torch.zeros(w["B"], device="cuda")
@@ -528,13 +657,14 @@ def main():
                      + 2 * w["B"] * w["H"] * w["M"] * w["D"] * 2 + w["B"] * w["H"] * w["N"] * 4)
         gbps = alg_bytes / stages[dom] * 1e-9
         roofline = {"kernel": dom, "bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                    "frac": gbps / PEAK_HBM_GBPS, "traffic": traffic, "algorithmic_bytes": alg_bytes,
-                    "avg_launch_ms": kernels[dom]["ms"]}
+                    "frac": gbps / PEAK_HBM_GBPS, "traffic": traffic, "traffic_source": traffic_source,
+                    "algorithmic_bytes": alg_bytes, "avg_launch_ms": kernels[dom]["ms"]}
     else:
         dom = "bwd_dkdv"
         roofline = {"kernel": dom, "bound": "mfma", "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
                     "unit": "TFLOP/s", "frac": kernels[dom]["tflops"] / PEAK_BF16_TFLOPS, "traffic": traffic,
-                    "algorithmic_flops": kern_flops[dom], "avg_launch_ms": kernels[dom]["ms"]}
+                    "traffic_source": traffic_source, "algorithmic_flops": kern_flops[dom],
+                    "avg_launch_ms": kernels[dom]["ms"]}
 
     line = {
         "metric": "fwd+bwd TFLOP/s & % bf16 MFMA peak, T=16k D=128; ACP speedup vs no-prune",
@@ -561,6 +691,11 @@ def main():
         line["decode"] = decode_report(max(5, ns.steps), 2)
         torch.cuda.empty_cache()
         line["head_dim_64"] = head_dim_report(max(2, ns.steps // 2), 1)
+        for name in ("c3d32", "c3d16"):
+            torch.cuda.empty_cache()
+            line["head_dim_" + name[3:]] = head_dim_report(max(2, ns.steps // 2), 1, name)
+        torch.cuda.empty_cache()
+        line["library_example"] = small_shape_report(ns.steps, ns.warmup)
     print(json.dumps(line))
 
 

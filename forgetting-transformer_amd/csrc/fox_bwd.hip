@@ -1,12 +1,17 @@
 // Backward kernels of Forgetting Attention for gfx950.
 //
-//   delta_kernel : delta_i = sum_d o_id * do_id
-//   dkdv_kernel  : one workgroup keeps 128 key rows (K, V in registers as MFMA B
-//                  operands; dK^T, dV^T accumulators) and walks the query tiles
-//                  below its diagonal; writes dk, dv and dc[n] = -sum_i dS[i,n].
 //   dq_kernel    : one workgroup keeps 128 query rows (Q, dO in registers) and
-//                  walks the key tiles like the forward; writes dq and adds
-//                  sum_j dS[i,j] into dc[i + N - M].
+//                  walks the key tiles like the forward; computes delta_i =
+//                  sum_d o_id * do_id for its rows on the way in, writes dq,
+//                  delta and the row sums drow[i] = sum_j dS[i,j].
+//   dkdv_kernel  : runs after it.  One workgroup keeps 128 key rows (K, V in
+//                  registers as MFMA B operands; dK^T, dV^T accumulators) and
+//                  walks the query tiles below its diagonal; writes dk, dv and
+//                  dc[n] = drow[n - (N - M)] - sum_i dS[i,n].
+//   delta_kernel : delta alone (a stage of its own for callers that want it;
+//                  the backward does not launch it).
+// Every kernel only stores: no read-modify-write of anything another kernel wrote,
+// so a stage may be repeated or timed alone without changing the result.
 //
 // Probabilities are rebuilt from the stored log-normaliser:
 //   P = exp2( (q.k)*sm_scale*log2e + rowc_i - colc_j ),
@@ -394,7 +399,12 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void dkdv_kernel(const BwdK a
   }
   wait_vmem_all();  // whatever was requested last (possibly an empty tile) has landed before the buffers are reused
   const float ctot = half_sum(csum);
-  if (n < N && g == 0) a.dc[(int64_t)bh * N + n] = -ctot;
+  // gradient w.r.t. the cumulative sum: the row sum the dQ kernel left for the query row that sits at this key
+  // position (none left of the first query row) minus this key's column sum
+  if (n < N && g == 0) {
+    const float rtot = n >= p_seq ? a.drow[(int64_t)bh * M + (n - p_seq)] : 0.f;
+    a.dc[(int64_t)bh * N + n] = rtot - ctot;
+  }
   // dK and dV leave through LDS (the tile buffers are free now) so that the global stores are whole rows
   static_assert(2 * kStoreStageBytes<D> <= Tile<D>::bytes(BMQ), "two waves stage in one tile buffer");
   __syncthreads();  // every wave is done with the tiles of the last step
@@ -471,6 +481,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
   const uint16_t* kp = a.k.ptr + b * a.k.sb + h * a.k.sh;
   const uint16_t* vp = a.v.ptr + b * a.v.sb + h * a.v.sh;
   const uint16_t* dop = a.d_o.ptr + b * a.d_o.sb + h * a.d_o.sh;
+  const uint16_t* op = a.o.ptr + b * a.o.sb + h * a.o.sh;
   uint16_t* dqp = const_cast<uint16_t*>(a.dq.ptr) + b * a.dq.sb + h * a.dq.sh;
 
   const int a0 = p_seq + m0;
@@ -499,10 +510,24 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
   const float c_ref = c_row[a0];
   // rows past M and empty rows (lse = -inf) get rowc = -inf through the subtraction: no load behind a branch
   const int mc = min(m, M - 1);
-  const float l = a.lse[(int64_t)bh * M + mc], c_m = c_row[min(p_seq + mc, N - 1)], dlt = a.delta[(int64_t)bh * M + mc];
+  const float l = a.lse[(int64_t)bh * M + mc], c_m = c_row[min(p_seq + mc, N - 1)];
   const float l_eff = ((m < M) & (l > -INFINITY)) ? l : INFINITY;
   const float rowc = (c_m - c_ref - l_eff) * kLog2e;
-  const float delta = m < M ? dlt : 0.f;
+  // delta_i = sum_d o_id * do_id (_bwd_preprocess of the reference, :902-943) for this lane's row: each half of
+  // the wave holds half of the row's elements.  Rows past M were loaded as zeros.  Stored for the dK/dV kernel.
+  float delta;
+  {
+    u32x4 oreg[KK];
+    load_row_operand_regs<D>(oreg, op, a.o.st, m, M, g);
+    float part = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        part += Tr::lo(oreg[kk][e]) * Tr::lo(doreg[kk][e]) + Tr::hi(oreg[kk][e]) * Tr::hi(doreg[kk][e]);
+    delta = half_sum(part);
+    if (m < M && g == 0) a.delta[(int64_t)bh * M + m] = delta;
+  }
 
   f32x16 dqacc[DB];
 #pragma unroll
@@ -564,7 +589,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
   }
 
   const float rtot = half_sum(rsum);
-  if (m < M && g == 0) a.dc[(int64_t)bh * N + a_m] += rtot;  // the dK/dV kernel wrote the column part earlier on this stream
+  if (m < M && g == 0) a.drow[(int64_t)bh * M + m] = rtot;  // the dK/dV kernel, next on this stream, folds it into dc
   // dQ leaves through LDS (the tile buffers are free now, one per wave) so that the global stores are whole rows
   static_assert(kStoreStageBytes<D> <= Tile<D>::bytes(BN), "one wave stages in one tile buffer");
   __syncthreads();  // every wave is done with the last tile

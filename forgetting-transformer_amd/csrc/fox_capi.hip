@@ -102,6 +102,7 @@ int make_bwd(const fox_bwd_args* args, fox::BwdK& k, bool need_grads) {
   k.o = to_view(args->o);
   k.d_o = to_view(args->d_o);
   k.delta = args->delta;
+  k.drow = args->delta + (int64_t)args->dims.B * args->dims.H * args->dims.M;
   k.B = args->dims.B; k.H = args->dims.H; k.M = args->dims.M; k.N = args->dims.N;
   k.sm_scale = args->sm_scale;
   k.n_tiles = 0;
@@ -375,9 +376,8 @@ int fox_attn_bwd_dq(const fox_bwd_args* args, void* stream) {
 int fox_attn_bwd(const fox_bwd_args* args, void* stream) {
   if (!args) return fail(FOX_E_ARG, "args is NULL");
   if (!args->dlog_fgate) return fail(FOX_E_ARG, "dlog_fgate is NULL");
-  FOX_TRY(fox_attn_bwd_delta(args, stream));
-  FOX_TRY(fox_attn_bwd_dkdv(args, stream));
   FOX_TRY(fox_attn_bwd_dq(args, stream));
+  FOX_TRY(fox_attn_bwd_dkdv(args, stream));
   return fox_cumsum_bwd(args->dlog_lambda, args->dlog_fgate, args->dims.B, args->dims.H, args->dims.N, stream);
 }
 

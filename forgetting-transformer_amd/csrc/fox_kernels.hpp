@@ -32,7 +32,8 @@ struct BwdK {
   const float* lse;
   const int64_t* seq_start;
   const float* thr;
-  float* delta;
+  float* delta;   // (B,H,M): rowsum(o * do), written by the dQ kernel
+  float* drow;    // (B,H,M): row sums of dS, written by the dQ kernel, read by the dK/dV kernel
   float* dc;
   int B, H, M, N;
   float sm_scale;

@@ -266,7 +266,7 @@ def _backward(ctx, do):
     do = maybe_contiguous(do)
     with torch.cuda.device(device):
         stream = _stream(device)
-        delta = torch.empty_like(L)
+        delta = torch.empty((2, B, H, M), dtype=torch.float32, device=device)   # rowsum(o * do), row sums of dS
         dlog_lambda = torch.empty((B, H, N), dtype=torch.float32, device=device)
         dlog_fgate = torch.empty((B, H, N), dtype=torch.float32, device=device) if gate_logit is None else None
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
@@ -281,9 +281,8 @@ def _backward(ctx, do):
             _lib.check(lib.fox_attn_bwd(C.byref(args), stream), "fox_attn_bwd")
             dgate = dlog_fgate
         else:  # same stages, the last one fused with the derivative of logsigmoid
-            _lib.check(lib.fox_attn_bwd_delta(C.byref(args), stream), "fox_attn_bwd_delta")
-            _lib.check(lib.fox_attn_bwd_dkdv(C.byref(args), stream), "fox_attn_bwd_dkdv")
             _lib.check(lib.fox_attn_bwd_dq(C.byref(args), stream), "fox_attn_bwd_dq")
+            _lib.check(lib.fox_attn_bwd_dkdv(C.byref(args), stream), "fox_attn_bwd_dkdv")
             dgate = torch.empty_like(gate_logit)
             _lib.check(lib.fox_gate_cumsum_bwd(_ptr(dlog_lambda), _ptr(gate_logit), _GATE_DTYPES[gate_logit.dtype],
                                                gate_logit.stride(0), gate_logit.stride(1), gate_logit.stride(2),

@@ -152,18 +152,23 @@ typedef struct fox_bwd_args {
   const int64_t* seq_start;   /* (B,) or NULL */
   const float* threshold;     /* (B,H) or NULL */
   float sm_scale;
-  float* delta;               /* (B,H,M) workspace, written */
+  float* delta;               /* (2,B,H,M) workspace, written: rowsum(o * do), then the row sums of dS */
   float* dlog_lambda;         /* (B,H,N) workspace, written: gradient w.r.t. c */
   float* dlog_fgate;          /* (B,H,N) written: gradient w.r.t. log_fgate */
 } fox_bwd_args;
 
 /*
- * The four stages of the backward pass, in the order they must run on a stream:
- *   fox_attn_bwd_delta : delta = rowsum(o * do)                     (_bwd_preprocess :902-943)
- *   fox_attn_bwd_dkdv  : dk, dv, dlog_lambda[n] = -sum_i dS[i,n]   (_find_end_index_kernel :747-795 + _bwd_kv_kernel :956-1143)
- *   fox_attn_bwd_dq    : dq, dlog_lambda[i+N-M] += sum_j dS[i,j]   (_find_start_index_kernel + _bwd_q_kernel :1156-1344)
+ * The stages of the backward pass, in the order they must run on a stream:
+ *   fox_attn_bwd_dq    : dq; delta = rowsum(o * do) and drow[i] = sum_j dS[i,j] into the two planes of `delta`
+ *                        (_bwd_preprocess :902-943 + _find_start_index_kernel + _bwd_q_kernel :1156-1344)
+ *   fox_attn_bwd_dkdv  : dk, dv, dlog_lambda[n] = drow[n-(N-M)] - sum_i dS[i,n]; reads both planes of `delta`
+ *                        (_find_end_index_kernel :747-795 + _bwd_kv_kernel :956-1143)
  *   fox_cumsum_bwd     : dlog_fgate from dlog_lambda                (:390-392)
- * fox_attn_bwd runs all four (ForgettingAttention.backward :232-400).
+ * fox_attn_bwd runs all three (ForgettingAttention.backward :232-400).  The reference launches the key/value
+ * kernel first and lets the query kernel add its row sums into the same buffer (:1334-1344); here every stage
+ * only stores, so repeating a stage (or timing it alone) leaves the result unchanged, and only the order
+ * dq before dkdv matters.  fox_attn_bwd_delta writes the first plane of `delta` alone (_bwd_preprocess as a stage
+ * of its own); the backward does not need it.
  */
 int fox_attn_bwd_delta(const fox_bwd_args* args, void* stream);
 int fox_attn_bwd_dkdv(const fox_bwd_args* args, void* stream);
