@@ -59,14 +59,16 @@ __global__ __launch_bounds__(256) void delta_kernel(const BwdK a) {
 }
 
 // ---------------------------------------------------------------------------
-// One step (kKvBM query rows) of the dK/dV kernel for one wave (32 key rows).
-// rc_s holds rowc_i / (sm_scale*log2e) and dl_s holds -delta_i.
-template <typename Tr, int D>
+// One step (BMQ query rows) of the dK/dV kernel for one wave (32 key rows).
+// rc_s holds rowc_i / (sm_scale*log2e) and dl_s holds -delta_i.  The wave accumulates the NDB 32-column
+// blocks of dK and dV that start at block db0 (all of them, or one half of the head dim when two waves
+// share a block of keys).
+template <typename Tr, int D, int BMQ = kKvBM, int NDB = (D + 31) / 32>
 __device__ __forceinline__ void dkdv_step(const char* q_tile, const char* do_tile, const float* rc_s, const float* dl_s,
-                                 const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16], f32x16 (&dkacc)[(D + 31) / 32],
-                                 f32x16 (&dvacc)[(D + 31) / 32], float& csum, int a_s0, int n, int n_w0, float qk_scale,
-                                 float colc, int lane) {
-  constexpr int BMQ = kKvBM, KK = D / 16, DB = (D + 31) / 32, MB = BMQ / 32;
+                                 const u32x4 (&kreg)[D / 16], const u32x4 (&vreg)[D / 16], f32x16 (&dkacc)[NDB],
+                                 f32x16 (&dvacc)[NDB], float& csum, int a_s0, int n, int n_w0, float qk_scale,
+                                 float colc, int lane, int db0 = 0) {
+  constexpr int KK = D / 16, MB = BMQ / 32;
   const int g = lane >> 5, i = lane & 31;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
@@ -94,9 +96,9 @@ __device__ __forceinline__ void dkdv_step(const char* q_tile, const char* do_til
       const u32x4 pb = pack8<Tr>(s, 8 * hh);
       const u32x4 dsb = pack8<Tr>(dp, 8 * hh);
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        dvacc[db] = Tr::mfma32(lds_col_operand<D>(do_tile, 32 * mb + 16 * hh, db, lane), pb, dvacc[db]);
-        dkacc[db] = Tr::mfma32(lds_col_operand<D>(q_tile, 32 * mb + 16 * hh, db, lane), dsb, dkacc[db]);
+      for (int db = 0; db < NDB; ++db) {
+        dvacc[db] = Tr::mfma32(lds_col_operand<D>(do_tile, 32 * mb + 16 * hh, db0 + db, lane), pb, dvacc[db]);
+        dkacc[db] = Tr::mfma32(lds_col_operand<D>(q_tile, 32 * mb + 16 * hh, db0 + db, lane), dsb, dkacc[db]);
       }
     }
   }
@@ -214,11 +216,16 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
   });
 }
 
-template <typename Tr, int D>
-__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void dkdv_kernel(const BwdK a) {
-  constexpr int BN = kKvBN, BMQ = kKvBM;
-  constexpr int KK = D / 16, DB = (D + 31) / 32;
-  static_assert(BN == 128, "four waves of 32 key rows");
+// DSPLIT: the variant for key tiles that pruning leaves a few query steps (class kClassLight).  Such a workgroup
+// is a short chain of loads, a few steps and stores; at one workgroup per CU nothing overlaps with it.  Here two
+// waves share 32 keys, each recomputing S and dP and accumulating one half of the head dim of dK and dV, so that
+// the kernel fits in 256 registers; a workgroup is 64 keys x 2 halves with query steps of 64 rows, and two
+// workgroups (two waves per SIMD) share a CU.
+template <typename Tr, int D, bool DSPLIT>
+__global__ __launch_bounds__(256, (D <= 64 || DSPLIT) ? 2 : 1) void dkdv_kernel(const BwdK a) {
+  constexpr int BN = DSPLIT ? 64 : kKvBN, BMQ = DSPLIT ? 64 : kKvBM;
+  constexpr int KK = D / 16, DB = (D + 31) / 32, NDB = DSPLIT ? DB / 2 : DB, DW = DSPLIT ? D / 2 : D;
+  static_assert(!DSPLIT || DB % 2 == 0, "the head dim splits into two halves of whole 32-column blocks");
   __shared__ __align__(16) char q_tile0[Tile<D>::bytes(BMQ)];
   __shared__ __align__(16) char q_tile1[Tile<D>::bytes(BMQ)];
   __shared__ __align__(16) char do_tile0[Tile<D>::bytes(BMQ)];
@@ -229,6 +236,8 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void dkdv_kernel(const BwdK a
   __shared__ __align__(16) float dl_s1[BMQ];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), g = lane >> 5, i = lane & 31;
+  const int kb = DSPLIT ? wave >> 1 : wave;   // block of 32 keys this wave owns
+  const int dh = DSPLIT ? wave & 1 : 0;       // half of the head dim it accumulates
   int bh, nt;
   decode_block(blockIdx.x, a.n_tiles, a.B * a.H, bh, nt);
   nt = a.n_tiles - 1 - nt;  // the first key tiles see the most query rows: start them first
@@ -236,6 +245,11 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void dkdv_kernel(const BwdK a
   const int M = a.M, N = a.N, p_seq = N - M;
   const int n0 = nt * BN;
   const float* c_row = a.c + (int64_t)bh * N;
+  if (a.cls != kClassAll) {  // the class of the 128-key tile this workgroup's keys belong to decides who handles them
+    const int n_last = min(N - 1, (n0 / kKvBN) * kKvBN + kKvBN - 1);
+    const bool light = acp_light_k(c_row, c_row[n_last], a.thr ? a.thr[bh] : 0.f, n_last, N, a.light_limit);
+    if (light != (a.cls == kClassLight)) return;
+  }
   const float* lse_row = a.lse + (int64_t)bh * M;
   const float* delta_row = a.delta + (int64_t)bh * M;
   const uint16_t* qp = a.q.ptr + b * a.q.sb + h * a.q.sh;
@@ -253,7 +267,7 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void dkdv_kernel(const BwdK a
   // query range: rows whose key position reaches this tile, up to the pruning bound
   int m_lo = max(n0 - p_seq, 0);
   m_lo = (m_lo / BMQ) * BMQ;
-  const int n_w0 = n0 + 32 * wave;
+  const int n_w0 = n0 + 32 * kb;
   const int n = n_w0 + i;  // this lane's key row
   // Everything the workgroup needs first is requested before anything is waited for: the tile of the
   // first diagonal step (it does not depend on the pruning bound), K and V, then the per-row terms.
@@ -302,9 +316,9 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void dkdv_kernel(const BwdK a
   if (early) issue_rows(m_lo);
   const float colc = (n < N && n >= seq) ? (c_key - c_ref) * kLog2e : INFINITY;
 
-  f32x16 dkacc[DB], dvacc[DB];
+  f32x16 dkacc[NDB], dvacc[NDB];
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+  for (int db = 0; db < NDB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
   float csum = 0.f;
@@ -338,23 +352,24 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void dkdv_kernel(const BwdK a
     wait_vmem_all();
     __syncthreads();
     if (t == n_diag - 1 && n_int > 0) issue(m_top, q_tile0, do_tile0);
-    dkdv_step<Tr, D>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane);
+    dkdv_step<Tr, D, BMQ, NDB>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc,
+                               lane, dh * NDB);
   }
   if (n_int > 0) {
     if (n_diag == 0) issue(m_top, q_tile0, do_tile0);
     if (row_lane) { rc_s0[row_slot] = rc_term(); dl_s0[row_slot] = dl_term(); }
   }
-  if constexpr (D <= 64) {
-    // Small head dims leave room for two workgroups per CU: the second wave on each SIMD fills the matrix pipe
-    // while the first does its vector work, so the plain step is used for interior tiles too.
+  if constexpr (D <= 64 || DSPLIT) {
+    // Small head dims (and the split variant) leave room for two workgroups per CU: the second wave on each SIMD
+    // fills the matrix pipe while the first does its vector work, so the plain step is used for interior tiles too.
     for (int t = 0; t < n_int; ++t) {
       const bool odd = t & 1;
       wait_vmem_all();
       __syncthreads();
       if (t + 1 < n_int) issue(m_top - (t + 1) * BMQ, odd ? q_tile0 : q_tile1, odd ? do_tile0 : do_tile1);
       const int ms = m_top - t * BMQ;
-      dkdv_step<Tr, D>(odd ? q_tile1 : q_tile0, odd ? do_tile1 : do_tile0, odd ? rc_s1 : rc_s0, odd ? dl_s1 : dl_s0, kreg, vreg,
-                       dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane);
+      dkdv_step<Tr, D, BMQ, NDB>(odd ? q_tile1 : q_tile0, odd ? do_tile1 : do_tile0, odd ? rc_s1 : rc_s0, odd ? dl_s1 : dl_s0, kreg,
+                                 vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane, dh * NDB);
       if (t + 1 < n_int && row_lane) {
         (odd ? rc_s0 : rc_s1)[row_slot] = rc_term();
         (odd ? dl_s0 : dl_s1)[row_slot] = dl_term();
@@ -401,16 +416,17 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void dkdv_kernel(const BwdK a
   const float ctot = half_sum(csum);
   // gradient w.r.t. the cumulative sum: the row sum the dQ kernel left for the query row that sits at this key
   // position (none left of the first query row) minus this key's column sum
-  if (n < N && g == 0) {
+  if (n < N && g == 0 && dh == 0) {  // (the two waves of a split pair hold the same column sums)
     const float rtot = n >= p_seq ? a.drow[(int64_t)bh * M + (n - p_seq)] : 0.f;
     a.dc[(int64_t)bh * N + n] = rtot - ctot;
   }
-  // dK and dV leave through LDS (the tile buffers are free now) so that the global stores are whole rows
-  static_assert(2 * kStoreStageBytes<D> <= Tile<D>::bytes(BMQ), "two waves stage in one tile buffer");
+  // dK and dV leave through LDS (the tile buffers are free now) so that the global stores are whole rows (of the
+  // wave's DW columns)
+  static_assert(2 * kStoreStageBytes<DW> <= Tile<D>::bytes(BMQ), "two waves stage in one tile buffer");
   __syncthreads();  // every wave is done with the tiles of the last step
-  char* stage = (wave < 2 ? q_tile0 : do_tile0) + (wave & 1) * kStoreStageBytes<D>;
-  store_rows_via_lds<Tr, D>(stage, dkacc, a.sm_scale, dkp, a.dk.st, n_w0, N, lane);
-  store_rows_via_lds<Tr, D>(stage, dvacc, 1.0f, dvp, a.dv.st, n_w0, N, lane);
+  char* stage = (wave < 2 ? q_tile0 : do_tile0) + (wave & 1) * kStoreStageBytes<DW>;
+  store_rows_via_lds<Tr, DW>(stage, dkacc, a.sm_scale, dkp + dh * DW, a.dk.st, n_w0, N, lane);
+  store_rows_via_lds<Tr, DW>(stage, dvacc, 1.0f, dvp + dh * DW, a.dv.st, n_w0, N, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -605,8 +621,14 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
   template __global__ void KERNEL<TR, 128>(const BwdK);
 FOX_INSTANTIATE_BWD(delta_kernel, Bf16)
 FOX_INSTANTIATE_BWD(delta_kernel, Fp16)
-FOX_INSTANTIATE_BWD(dkdv_kernel, Bf16)
-FOX_INSTANTIATE_BWD(dkdv_kernel, Fp16)
+#define FOX_INSTANTIATE_DKDV(TR)                                     \
+  template __global__ void dkdv_kernel<TR, 16, false>(const BwdK);   \
+  template __global__ void dkdv_kernel<TR, 32, false>(const BwdK);   \
+  template __global__ void dkdv_kernel<TR, 64, false>(const BwdK);   \
+  template __global__ void dkdv_kernel<TR, 128, false>(const BwdK);  \
+  template __global__ void dkdv_kernel<TR, 128, true>(const BwdK);
+FOX_INSTANTIATE_DKDV(Bf16)
+FOX_INSTANTIATE_DKDV(Fp16)
 FOX_INSTANTIATE_BWD(dq_kernel, Bf16)
 FOX_INSTANTIATE_BWD(dq_kernel, Fp16)
 
@@ -629,9 +651,21 @@ static hipError_t delta_t(const BwdK& a, int D, hipStream_t s) {
 template <typename Tr>
 static hipError_t dkdv_t(const BwdK& a0, int D, hipStream_t s) {
   BwdK a = a0;
+  if (a.cls == kClassLight) {  // the split variant: 64 keys per workgroup
+    if (!dkdv_split_supports(D)) return hipErrorInvalidValue;
+    a.n_tiles = (a.N + 63) / 64;
+    hipLaunchKernelGGL((dkdv_kernel<Tr, 128, true>), dim3((unsigned)(a.n_tiles * a.B * a.H)), dim3(256), 0, s, a);
+    return hipGetLastError();
+  }
   a.n_tiles = (a.N + kKvBN - 1) / kKvBN;
   const dim3 grid((unsigned)(a.n_tiles * a.B * a.H));
-  FOX_DISPATCH_D(dkdv_kernel, grid, 0)
+  switch (D) {
+    case 16: hipLaunchKernelGGL((dkdv_kernel<Tr, 16, false>), grid, dim3(256), 0, s, a); break;
+    case 32: hipLaunchKernelGGL((dkdv_kernel<Tr, 32, false>), grid, dim3(256), 0, s, a); break;
+    case 64: hipLaunchKernelGGL((dkdv_kernel<Tr, 64, false>), grid, dim3(256), 0, s, a); break;
+    case 128: hipLaunchKernelGGL((dkdv_kernel<Tr, 128, false>), grid, dim3(256), 0, s, a); break;
+    default: return hipErrorInvalidValue;
+  }
   return hipGetLastError();
 }
 template <typename Tr>
@@ -642,6 +676,8 @@ static hipError_t dq_t(const BwdK& a0, int D, hipStream_t s) {
   FOX_DISPATCH_D(dq_kernel, grid, 0)
   return hipGetLastError();
 }
+
+bool dkdv_split_supports(int D) { return D == 128; }
 
 hipError_t launch_bwd_delta(const BwdK& a, int D, int dtype, hipStream_t s) {
   return dtype == 0 ? delta_t<Bf16>(a, D, s) : delta_t<Fp16>(a, D, s);

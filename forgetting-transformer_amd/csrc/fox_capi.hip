@@ -7,8 +7,10 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <mutex>
 
+#include "fox_common.hpp"
 #include "fox_kernels.hpp"
 
 // Library-owned scratch of fox_attn_fwd_noalloc: the partial (max, sum, accumulator) results of a key-split
@@ -61,6 +63,25 @@ int check_extent(const fox_view* v, int rows, int D, const char* name) {
   const int64_t bytes = ((int64_t)(rows - 1) * v->stride_t + D) * 2;
   if (v->stride_t <= 0 || bytes >= (int64_t)1 << 31) return fail(FOX_E_ARG, "%s: one (batch, head) slice must span less than 2 GiB with a positive row stride", name);
   return FOX_OK;
+}
+
+// Distance from the diagonal, in keys, within which the pruning bound of a 128-key tile must lie for the tile to go
+// to the split variant of the dK/dV kernel (fox_set_acp_light_limit): 0 = never, negative = every tile of every
+// call that the variant supports.
+std::atomic<int> g_light_limit{256};   // measured crossover of the two kernels at head dim 128
+
+// The tile classes of a call: *first and *second are the classes of the launches to make (kClassAll alone,
+// kClassLight alone, or kClassLight then kClassHeavy), *limit the distance handed to the kernels.
+void tile_classes(bool pruned, bool light_ok, int* first, int* second, int* limit) {
+  const int lim = g_light_limit.load(std::memory_order_relaxed);
+  *first = fox::kClassAll;
+  *second = -1;
+  *limit = lim;
+  if (!light_ok || lim == 0) return;
+  if (lim < 0) { *first = fox::kClassLight; return; }
+  if (!pruned) return;
+  *first = fox::kClassLight;
+  *second = fox::kClassHeavy;
 }
 
 // Device address of `scratch` on the current device, looked up once per device.
@@ -237,6 +258,8 @@ int fox_version(void) { return 100; }  // 0.1.0
 
 const char* fox_last_error(void) { return g_err; }
 
+int32_t fox_set_acp_light_limit(int32_t keys) { return g_light_limit.exchange(keys, std::memory_order_relaxed); }
+
 int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_block_n, int32_t* kv_block_m) {
   if (D != 16 && D != 32 && D != 64 && D != 128) return fail(FOX_E_ARG, "head dim must be one of 16, 32, 64, 128 (got %d)", D);
   if (block_m) *block_m = fox::kFwdBM;
@@ -362,6 +385,12 @@ int fox_attn_bwd_dkdv(const fox_bwd_args* args, void* stream) {
   FOX_TRY(check_view(&args->dv, "dv"));
   k.dk = to_view(args->dk);
   k.dv = to_view(args->dv);
+  int first, second;
+  tile_classes(k.thr != nullptr, fox::dkdv_split_supports(args->dims.D), &first, &second, &k.light_limit);
+  k.cls = first;
+  FOX_TRY(check_hip(fox::launch_bwd_dkdv(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), "fox_attn_bwd_dkdv"));
+  if (second < 0) return FOX_OK;
+  k.cls = second;
   return check_hip(fox::launch_bwd_dkdv(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), "fox_attn_bwd_dkdv");
 }
 

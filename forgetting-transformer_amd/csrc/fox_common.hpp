@@ -364,6 +364,20 @@ __device__ __forceinline__ int acp_first_kept_block(const float* c_row, float c_
   return first;
 }
 
+// Classes of key tiles in the dK/dV pass under pruning.  A launch of class kClassLight handles only the 128-key
+// tiles whose pruning bound lies within `limit` positions of their diagonal, a launch of class kClassHeavy only
+// the others; both evaluate the same predicate, so every tile is handled exactly once.  limit < 0 names every
+// tile light.
+constexpr int kClassAll = 0, kClassLight = 1, kClassHeavy = 2;
+
+// Key tile whose last key is at position n_last (c_last = c[n_last]): light when the query row that sits
+// `limit` positions after n_last is already below the threshold against that key (c is non-increasing, so
+// every later row is too), or when there is no such row.
+__device__ __forceinline__ bool acp_light_k(const float* c_row, float c_last, float thr, int n_last, int N, int limit) {
+  if (limit < 0 || n_last + limit >= N) return true;
+  return (c_row[n_last + limit] - c_last) < thr;
+}
+
 // Key-side bound: the first query block (BMQ rows, first row u*BMQ) in [u_lo, U)
 // whose largest decay against the key tile,  c[P_SEQ + u*BMQ] - c_last,  is below
 // thr; every later block is prunable too.  Returns U when none is.

@@ -38,6 +38,8 @@ struct BwdK {
   int B, H, M, N;
   float sm_scale;
   int n_tiles;
+  int cls;         // kClassAll, or the class of key tiles this dK/dV launch handles (fox_common.hpp)
+  int light_limit; // distance from the diagonal, in keys, that separates the two classes
 };
 
 // Token shift: x, out, dout, dx are (B, T, H, D) 16-bit with shared element strides; the weights and
@@ -83,7 +85,8 @@ constexpr int kKvBM = 128;   // query rows per step in the dK/dV kernel
 hipError_t launch_fwd(const FwdK& a, int D, int dtype, hipStream_t s);
 int fwd_key_splits(int B, int H, int M, int N);
 hipError_t launch_bwd_delta(const BwdK& a, int D, int dtype, hipStream_t s);
-hipError_t launch_bwd_dkdv(const BwdK& a, int D, int dtype, hipStream_t s);
+hipError_t launch_bwd_dkdv(const BwdK& a, int D, int dtype, hipStream_t s);   // a.cls selects the variant and its tiles
+bool dkdv_split_supports(int D);   // head dims the split (kClassLight) variant of the dK/dV kernel exists for
 hipError_t launch_bwd_dq(const BwdK& a, int D, int dtype, hipStream_t s);
 hipError_t launch_fwd_decode(const FwdK& a, int D, int dtype, hipStream_t s);  // M == 1, without the merge of the splits
 hipError_t launch_norm_gate(const NormGateK& a, int D, int dtype, bool bwd, int act, hipStream_t s);  // act: FOX_ACT_*

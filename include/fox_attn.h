@@ -57,6 +57,17 @@ const char* fox_last_error(void);
 int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_block_n, int32_t* kv_block_m);
 
 /*
+ * Under pruning the dK/dV pass is served by two kernels: 128-key tiles whose pruning bound lies within `keys`
+ * positions of their diagonal (a few query steps: a short chain of loads and stores) go to a variant that
+ * splits the head dim over two waves and runs two workgroups per CU, the others to the kernel built for long
+ * loops.  This sets `keys` (256 by default, the measured crossover) for all later calls of the process and returns the previous value: 0 = the long-loop
+ * kernel only, negative = the split variant for every tile of every call it supports (head dim 128), with or
+ * without a threshold.  The results obey the same contract either way.  Like the reference's tile pickers,
+ * which "can be overwritten at runtime" (get_bwd_kv_config, :838).
+ */
+int32_t fox_set_acp_light_limit(int32_t keys);
+
+/*
  * c[b,h,n] = sum_{l<=n} g[b,h,l] with g[b,h,l] taken as 0 for l < seq_start[b].
  * g is fp32 with element strides (g_sb, g_sh, g_sn); c is (B,H,N) contiguous fp32.
  * seq_start may be NULL.  Replaces the prologue at :117-127 (clone, masked zero

@@ -253,6 +253,25 @@ def test_log_normalizer_and_start_index_outputs(fa):
     assert si.dtype == torch.long and si.shape == (2, 3, 3)
 
 
+@pytest.mark.parametrize("limit", [-1, 0, 64])
+@pytest.mark.parametrize("B,H,M,N,seq,thr,gates", [
+    (1, 3, 129, 129, None, None, (0.0, 1.0)), (2, 2, 200, 457, [5, 300], None, (0.0, 1.0)), (1, 2, 940, 940, None, -6.0, (0.0, 1.0)),
+    (2, 2, 700, 950, None, -10.0, (-1.0, 2.0)), (1, 2, 5, 5, None, None, (0.0, 1.0)), (1, 1, 127, 257, [200], "auto", (1.0, 1.0)),
+    (2, 4, 2048, 2048, [0, 1024], -20.0, (2.0, 1.0)), (2, 2, 1000, 3000, None, -20.0, (1.0, 1.0)), (1, 2, 1, 300, None, None, (0.0, 1.0))])
+def test_dkdv_kernel_variants(fa, limit, B, H, M, N, seq, thr, gates):
+    """The dK/dV pass at head dim 128 has two kernels (long loops; head dim split over two waves for key tiles pruned
+    down to a few steps) and a per-tile choice between them.  Every tile through the split variant (-1, with and
+    without a threshold), none (0), and a mix decided tile by tile (64 keys): all against the oracle."""
+    from forgetting_transformer.ops import _lib
+    lib = _lib.load()
+    prev = lib.fox_set_acp_light_limit(limit)
+    try:
+        tol = REL_TOL + (4.0 * N * math.exp(thr) if isinstance(thr, float) else 0.0)
+        run_case(fa, B, H, M, N, 128, seq_start=seq, thr=thr, tol=tol, gate_mean=gates[0], gate_std=gates[1], seed=M + N, qkv_std=0.7)
+    finally:
+        assert lib.fox_set_acp_light_limit(prev) == limit
+
+
 def test_in_op_timers_fill_the_info_table(fa):
     """The reference's hidden timing flags (:45-70, :176-181, :217-222): same results, and the class-level table
     gets the elapsed milliseconds and call counts under the caller's key."""
