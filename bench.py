@@ -211,7 +211,7 @@ def stage_times(w, tensors, iters, threshold=None):
     for name, fn in (("bwd_dq", lib.fox_attn_bwd_dq), ("bwd_dkdv", lib.fox_attn_bwd_dkdv)):
         out[name] = event_time(lambda fn=fn, name=name: _lib.check(fn(C.byref(bwd), stream), name), iters)
     out["cumsum_bwd"] = event_time(
-        lambda: _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg.data_ptr(), B, H, N, stream), "cumsum_bwd"), iters)
+        lambda: _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg.data_ptr(), 0, 0, 0, B, H, N, stream), "cumsum_bwd"), iters)
     return out
 
 
@@ -400,8 +400,8 @@ def small_shape_report(steps, warmup):
     def step():
         forgetting_attention(q, k, v, log_fgate).backward(dout)
         q.grad = k.grad = v.grad = log_fgate.grad = None
-    t = time_steps(step, max(steps, 50), max(warmup, 5))
-    t_graph = graph_time(step, max(steps, 50))
+    t = time_steps(step, max(steps, 300), max(warmup, 30))
+    t_graph = graph_time(step, max(steps, 300))
     st = stage_times(w, tensors, max(steps, 20))
     path = ("cumsum_fwd", "fwd", "bwd_dq", "bwd_dkdv", "cumsum_bwd")
     return {"workload": "B4 T512 H12 D64 bf16 fwd+bwd, gate logits N(0,1)", "wall_ms_per_step": t * 1e3,

@@ -328,11 +328,13 @@ int fox_gate_cumsum_bwd(const float* dc, const void* logits, int32_t logits_dtyp
                    "fox_gate_cumsum_bwd");
 }
 
-int fox_cumsum_bwd(const float* dc, float* dg, int32_t B, int32_t H, int32_t N, void* stream) {
+int fox_cumsum_bwd(const float* dc, float* dg, int64_t dg_sb, int64_t dg_sh, int64_t dg_sn, int32_t B, int32_t H, int32_t N,
+                   void* stream) {
   if (!dc || !dg) return fail(FOX_E_ARG, "dc and dg must not be NULL");
   if (B <= 0 || H <= 0 || N <= 0) return fail(FOX_E_ARG, "B, H, N must be positive");
   if (dc == dg) return fail(FOX_E_ARG, "dc and dg must not alias");
-  return check_hip(fox::launch_cumsum_bwd(dc, dg, B, H, N, (hipStream_t)stream), "fox_cumsum_bwd");
+  if (dg_sb == 0 && dg_sh == 0 && dg_sn == 0) { dg_sb = (int64_t)H * N; dg_sh = N; dg_sn = 1; }   // contiguous (B,H,N)
+  return check_hip(fox::launch_cumsum_bwd(dc, dg, dg_sb, dg_sh, dg_sn, B, H, N, (hipStream_t)stream), "fox_cumsum_bwd");
 }
 
 int fox_auto_threshold(const fox_dims* dims, const fox_view* q, const fox_view* k, float sm_scale, float* thr,
@@ -407,7 +409,8 @@ int fox_attn_bwd(const fox_bwd_args* args, void* stream) {
   if (!args->dlog_fgate) return fail(FOX_E_ARG, "dlog_fgate is NULL");
   FOX_TRY(fox_attn_bwd_dq(args, stream));
   FOX_TRY(fox_attn_bwd_dkdv(args, stream));
-  return fox_cumsum_bwd(args->dlog_lambda, args->dlog_fgate, args->dims.B, args->dims.H, args->dims.N, stream);
+  return fox_cumsum_bwd(args->dlog_lambda, args->dlog_fgate, args->dlog_fgate_stride_b, args->dlog_fgate_stride_h,
+                        args->dlog_fgate_stride_n, args->dims.B, args->dims.H, args->dims.N, stream);
 }
 
 }  // extern "C"

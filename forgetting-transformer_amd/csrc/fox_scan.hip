@@ -92,11 +92,11 @@ __device__ __forceinline__ void scan_row(int N, Load load, Store store) {
 
 template <bool REVERSE>
 __global__ __launch_bounds__(kScanThreads) void scan_kernel(const float* __restrict__ in, int64_t sb, int64_t sh, int64_t sn,
-                                                   const int64_t* __restrict__ seq_start, float* __restrict__ out, int H,
-                                                   int N) {
+                                                   const int64_t* __restrict__ seq_start, float* __restrict__ out, int64_t ob,
+                                                   int64_t oh, int64_t on, int H, int N) {
   const int bh = blockIdx.x, b = bh / H, h = bh % H;
   const float* src = in + b * sb + h * sh;
-  float* dst = out + (int64_t)bh * N;
+  float* dst = out + b * ob + h * oh;
   int seq = 0;
   if (!REVERSE && seq_start) {
     const int64_t s64 = seq_start[b];
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(const float* __restr
   }
   scan_row<REVERSE>(
       N, [&](int idx) { return (REVERSE || idx >= seq) ? src[(int64_t)idx * sn] : 0.f; },
-      [&](int idx, float sum) { dst[idx] = sum; });
+      [&](int idx, float sum) { dst[(int64_t)idx * on] = sum; });
 }
 
 // Forget-gate logits in fp32, bf16 or fp16 (the output of the gate projection of the FoX layer).
@@ -206,13 +206,14 @@ hipError_t launch_gate_cumsum_bwd(const float* dc, const void* logits, int dtype
 
 hipError_t launch_cumsum_fwd(const float* g, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start, float* c, int B,
                              int H, int N, hipStream_t s) {
-  hipLaunchKernelGGL(scan_kernel<false>, dim3((unsigned)(B * H)), dim3(kScanThreads), 0, s, g, sb, sh, sn, seq_start, c, H, N);
+  hipLaunchKernelGGL(scan_kernel<false>, dim3((unsigned)(B * H)), dim3(kScanThreads), 0, s, g, sb, sh, sn, seq_start, c,
+                     (int64_t)H * N, (int64_t)N, (int64_t)1, H, N);
   return hipGetLastError();
 }
 
-hipError_t launch_cumsum_bwd(const float* dc, float* dg, int B, int H, int N, hipStream_t s) {
+hipError_t launch_cumsum_bwd(const float* dc, float* dg, int64_t db, int64_t dh, int64_t dn, int B, int H, int N, hipStream_t s) {
   hipLaunchKernelGGL(scan_kernel<true>, dim3((unsigned)(B * H)), dim3(kScanThreads), 0, s, dc, (int64_t)H * N, (int64_t)N, (int64_t)1,
-                     (const int64_t*)nullptr, dg, H, N);
+                     (const int64_t*)nullptr, dg, db, dh, dn, H, N);
   return hipGetLastError();
 }
 

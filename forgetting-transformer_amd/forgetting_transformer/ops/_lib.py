@@ -53,6 +53,7 @@ class BwdArgs(C.Structure):
         ("delta", C.c_void_p),
         ("dlog_lambda", C.c_void_p),
         ("dlog_fgate", C.c_void_p),
+        ("dlog_fgate_stride_b", C.c_int64), ("dlog_fgate_stride_h", C.c_int64), ("dlog_fgate_stride_n", C.c_int64),
     ]
 
 
@@ -106,7 +107,7 @@ SIGNATURES = {
     "fox_tile_config": (C.c_int, [C.c_int32] + [C.POINTER(C.c_int32)] * 4),
     "fox_cumsum_fwd": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                  C.c_int32, C.c_void_p]),
-    "fox_cumsum_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
+    "fox_cumsum_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "fox_gate_cumsum_fwd": (C.c_int, [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "fox_gate_cumsum_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int64,

@@ -13,6 +13,7 @@ call raises.
 from __future__ import annotations
 
 import ctypes as C
+import functools
 import math
 from collections import defaultdict
 from typing import Literal, Optional, Union
@@ -38,12 +39,40 @@ def maybe_contiguous(x: torch.Tensor) -> torch.Tensor:
     return x if ok else x.contiguous()
 
 
+def _is_dense(shape, strides) -> bool:
+    """True when the strides describe a permutation of a contiguous tensor (no gaps, no overlap)."""
+    expect = 1
+    for size, stride in sorted(zip(shape, strides), key=lambda p: p[1]):
+        if size == 1:
+            continue
+        if stride != expect:
+            return False
+        expect *= size
+    return True
+
+
 def _view(x: torch.Tensor) -> _lib.View:
     return _lib.View(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2))
 
 
 def _ptr(x: Optional[torch.Tensor]):
     return None if x is None else C.c_void_p(x.data_ptr())
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(device: torch.device):
+    """Context that makes ``device`` current; nothing to do (and nothing to pay) when it already is."""
+    return _NO_SWITCH if torch.cuda.current_device() == device.index else torch.cuda.device(device)
 
 
 def _stream(device: torch.device):
@@ -136,6 +165,22 @@ class ForgettingAttentionFromLogits(torch.autograd.Function):
 _GATE_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16, torch.float32: _lib.DTYPE_FP32}
 
 
+@functools.lru_cache(maxsize=256)
+def _fwd_workspace_bytes(B, H, M, N, D, dtype_code):
+    """Bytes of key-split scratch the forward wants for a shape (0 = the shape is not split); asked once per shape."""
+    need = C.c_int64(0)
+    _lib.check(_lib.load().fox_attn_fwd_workspace_bytes(C.byref(_lib.Dims(B, H, M, N, D, dtype_code)), C.byref(need)),
+               "fox_attn_fwd_workspace_bytes")
+    return need.value
+
+
+@functools.lru_cache(maxsize=64)
+def _constant_threshold(value, B, H, device):
+    """(B, H) fp32 tensor holding one float threshold: the same values as as_tensor + broadcast_to of the reference
+    (:104-109), filled on the device once per (value, shape, device) instead of once per call.  Read-only."""
+    return torch.full((B, H), value, dtype=torch.float, device=device)
+
+
 def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
              return_log_normalizer, return_start_index):
     assert causal, "Only causal attention is supported"
@@ -173,7 +218,7 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
             auto_threshold = True
         elif isinstance(adaptive_threshold, (int, float)):
             # same values as as_tensor + broadcast_to below, filled on the device: no host-to-device copy to wait for
-            adaptive_threshold = torch.full((B, H), float(adaptive_threshold), dtype=torch.float, device=q.device)
+            adaptive_threshold = _constant_threshold(float(adaptive_threshold), B, H, q.device)
         else:
             adaptive_threshold = torch.as_tensor(adaptive_threshold, dtype=torch.float, device=q.device)
             try:
@@ -202,7 +247,7 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
 
     q, k, v = maybe_contiguous(q), maybe_contiguous(k), maybe_contiguous(v)
 
-    with torch.cuda.device(device):
+    with _on_device(device):
         stream = _stream(device)
 
         if auto_threshold:
@@ -212,8 +257,15 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
             _lib.check(lib.fox_auto_threshold(C.byref(dims), C.byref(qv), C.byref(kv), sm_scale,
                                               _ptr(adaptive_threshold), _ptr(scratch), stream), "fox_auto_threshold")
 
+        # log_lambda (B,H,N), the log-normaliser L (B,H,M) and the key-split scratch come from one allocation
+        ws_bytes = _fwd_workspace_bytes(B, H, M, N, D, dims.dtype)
+        n_c, n_l = (B * H * N + 3) // 4 * 4, (B * H * M + 3) // 4 * 4    # floats; the scratch behind them stays 16-byte aligned
+        buf = torch.empty(n_c + n_l + ws_bytes // 4, dtype=torch.float32, device=device)
+        log_lambda = buf[:B * H * N].view(B, H, N)
+        L = buf[n_c:n_c + B * H * M].view(B, H, M)
+        workspace = buf[n_c + n_l:] if ws_bytes > 0 else None
+
         # c = cumsum(log_fgate) with gates left of seq_start zeroed, one fused kernel
-        log_lambda = torch.empty((B, H, N), dtype=torch.float32, device=device)
         if gate_is_logit:  # logsigmoid fused into the scan; the fp32 log gates are a by-product
             ctx.log_fgate = torch.empty((B, H, N), dtype=torch.float32, device=device)
             _lib.check(lib.fox_gate_cumsum_fwd(_ptr(log_fgate), _GATE_DTYPES[log_fgate.dtype], log_fgate.stride(0),
@@ -226,19 +278,15 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
                        "fox_cumsum_fwd")
 
         o = torch.empty_like(q)
-        L = torch.empty((B, H, M), device=device, dtype=torch.float32)
         first_block = None
         if return_start_index:
             block_m, _, _, _ = _lib.tile_config(D)
             first_block = torch.zeros((B, H, (M + block_m - 1) // block_m), dtype=torch.int32, device=device)
-        ws_bytes = C.c_int64(0)
-        _lib.check(lib.fox_attn_fwd_workspace_bytes(C.byref(dims), C.byref(ws_bytes)), "fox_attn_fwd_workspace_bytes")
-        workspace = torch.empty(ws_bytes.value, dtype=torch.uint8, device=device) if ws_bytes.value > 0 else None
         args = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), log_lambda.data_ptr(), L.data_ptr(),
                             None if seq_start is None else seq_start.data_ptr(),
                             None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
                             sm_scale, None if first_block is None else first_block.data_ptr(),
-                            None if workspace is None else workspace.data_ptr(), ws_bytes.value)
+                            None if workspace is None else workspace.data_ptr(), ws_bytes)
         _lib.check(lib.fox_attn_fwd(C.byref(args), stream), "fox_attn_fwd")
 
     ctx.save_for_backward(q, k, v, o, L, log_lambda, seq_start, adaptive_threshold,
@@ -246,6 +294,7 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
     ctx.sm_scale = sm_scale
     ctx.causal = causal
     ctx.has_seq_start = has_seq_start
+    ctx.gate_strides = tuple(log_fgate.stride())
 
     if return_log_normalizer or return_start_index:
         start_index = None
@@ -264,11 +313,17 @@ def _backward(ctx, do):
     device = q.device
     lib = _lib.load()
     do = maybe_contiguous(do)
-    with torch.cuda.device(device):
+    with _on_device(device):
         stream = _stream(device)
-        delta = torch.empty((2, B, H, M), dtype=torch.float32, device=device)   # rowsum(o * do), row sums of dS
-        dlog_lambda = torch.empty((B, H, N), dtype=torch.float32, device=device)
-        dlog_fgate = torch.empty((B, H, N), dtype=torch.float32, device=device) if gate_logit is None else None
+        # one allocation for the fp32 temporaries: rowsum(o * do) and the row sums of dS (2,B,H,M), then dlog_lambda (B,H,N)
+        tmp = torch.empty(2 * B * H * M + B * H * N, dtype=torch.float32, device=device)
+        delta, dlog_lambda = tmp[:2 * B * H * M], tmp[2 * B * H * M:]
+        dlog_fgate = None
+        if gate_logit is None:
+            # in the layout of the caller's log_fgate when that is a permuted dense tensor (the (B,H,T) view of
+            # (B,T,H) memory the FoX layer passes): autograd then takes the gradient as it is, without a copy
+            gs = ctx.gate_strides if _is_dense((B, H, N), ctx.gate_strides) else (H * N, N, 1)
+            dlog_fgate = torch.empty_strided((B, H, N), gs, dtype=torch.float32, device=device)
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         args = _lib.BwdArgs(
             _lib.Dims(B, H, M, N, D, _DTYPES[q.dtype]),
@@ -276,7 +331,8 @@ def _backward(ctx, do):
             log_lambda.data_ptr(), L.data_ptr(),
             None if seq_start is None else seq_start.data_ptr(),
             None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
-            ctx.sm_scale, delta.data_ptr(), dlog_lambda.data_ptr(), None if dlog_fgate is None else dlog_fgate.data_ptr())
+            ctx.sm_scale, delta.data_ptr(), dlog_lambda.data_ptr(), None if dlog_fgate is None else dlog_fgate.data_ptr(),
+            *(dlog_fgate.stride() if dlog_fgate is not None else (0, 0, 0)))
         if gate_logit is None:
             _lib.check(lib.fox_attn_bwd(C.byref(args), stream), "fox_attn_bwd")
             dgate = dlog_fgate

@@ -77,10 +77,12 @@ int fox_cumsum_fwd(const float* g, int64_t g_sb, int64_t g_sh, int64_t g_sn, con
                    int32_t B, int32_t H, int32_t N, void* stream);
 
 /*
- * dg[b,h,l] = sum_{n>=l} dc[b,h,n]; both (B,H,N) contiguous fp32.
- * Replaces the reverse cumulative sum at :390-392.
+ * dg[b,h,l] = sum_{n>=l} dc[b,h,n]; dc is (B,H,N) contiguous fp32, dg is fp32 with element strides
+ * (dg_sb, dg_sh, dg_sn) -- the layout of the caller's log_fgate, so that autograd can take the gradient as it
+ * is -- or (B,H,N) contiguous when all three strides are 0.  Replaces the reverse cumulative sum at :390-392.
  */
-int fox_cumsum_bwd(const float* dc, float* dg, int32_t B, int32_t H, int32_t N, void* stream);
+int fox_cumsum_bwd(const float* dc, float* dg, int64_t dg_sb, int64_t dg_sh, int64_t dg_sn, int32_t B, int32_t H,
+                   int32_t N, void* stream);
 
 /*
  * The prologue of the FoX layer fused with the scan: c[b,h,n] = sum_{seq_start[b] <= l <= n} logsigmoid(x[b,h,l])
@@ -166,6 +168,7 @@ typedef struct fox_bwd_args {
   float* delta;               /* (2,B,H,M) workspace, written: rowsum(o * do), then the row sums of dS */
   float* dlog_lambda;         /* (B,H,N) workspace, written: gradient w.r.t. c */
   float* dlog_fgate;          /* (B,H,N) written: gradient w.r.t. log_fgate */
+  int64_t dlog_fgate_stride_b, dlog_fgate_stride_h, dlog_fgate_stride_n;  /* its element strides; all 0 = contiguous */
 } fox_bwd_args;
 
 /*

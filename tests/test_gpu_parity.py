@@ -340,9 +340,13 @@ def test_cumsum_kernels(fa):
     assert (c[1, :, :1234] == 0).all()
     dc = torch.randn(B, H, N, device="cuda")
     dg = torch.empty_like(dc)
-    _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg.data_ptr(), B, H, N, stream), "cumsum_bwd")
+    _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg.data_ptr(), 0, 0, 0, B, H, N, stream), "cumsum_bwd")
     ref = torch.flip(torch.cumsum(torch.flip(dc.double(), [-1]), -1), [-1])
     assert (dg.double() - ref).abs().max() <= 1e-6 * ref.abs().max()
+    # the same into a (B,H,N) view of (B,N,H) memory, the layout of the FoX layer's gates: bit for bit the same values
+    dg_t = torch.full((B, N, H), float("nan"), device="cuda").transpose(1, 2)
+    _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg_t.data_ptr(), *dg_t.stride(), B, H, N, stream), "cumsum_bwd")
+    assert torch.equal(dg_t, dg)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
