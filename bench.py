@@ -148,7 +148,7 @@ def event_time(fn, iters, warmup=2):
 
 def stage_times(w, tensors, iters, threshold=None):
     """Time every kernel of the path alone through the C ABI (launches go to torch's current stream).
-    threshold: optional pruning threshold (a float) applied to every (batch, head)."""
+    threshold: optional pruning threshold, a float applied to every (batch, head) or a (B, H) fp32 tensor."""
     from forgetting_transformer.ops import _lib
     from forgetting_transformer.ops.forgetting_attention import _view
 
@@ -171,7 +171,8 @@ def stage_times(w, tensors, iters, threshold=None):
     ws = torch.empty(max(ws_bytes.value, 16), dtype=torch.uint8, device=dev)  # key-split partials (prefill / decode shapes)
     thr = None
     if threshold is not None:
-        thr_t = torch.full((B, H), float(threshold), dtype=torch.float32, device=dev)
+        thr_t = (threshold if torch.is_tensor(threshold)
+                 else torch.full((B, H), float(threshold), dtype=torch.float32, device=dev))
         thr = thr_t.data_ptr()
     fwd = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), c.data_ptr(), lse.data_ptr(), ss, thr,
                        1.0 / math.sqrt(D), None, ws.data_ptr() if ws_bytes.value else None, ws_bytes.value)
@@ -591,6 +592,9 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift", "norm_gate", "ref_sweep"])
+    ap.add_argument("--threshold", default=None,
+                    help="adaptive_threshold of the main workload: a float or 'auto' (default: no pruning); with it the "
+                         "roofline entry prices the dK/dV pass against HBM, the bound of a heavily pruned step")
     ap.add_argument("--no-extras", action="store_true", help="skip the ACP and chunked-prefill reports")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -624,13 +628,15 @@ def main():
     q, k, v, log_fgate, dout, seq_start = tensors
     if not w["fwd_only"]:
         q, k, v, log_fgate = (x.requires_grad_() for x in (q, k, v, log_fgate))
+    thr = None if ns.threshold is None else ("auto" if ns.threshold == "auto" else float(ns.threshold))
 
     def step():
         if w["fwd_only"]:
             with torch.no_grad():
-                forgetting_attention(q, k, v, log_fgate, head_first=w["head_first"], seq_start=seq_start)
+                forgetting_attention(q, k, v, log_fgate, head_first=w["head_first"], seq_start=seq_start, adaptive_threshold=thr)
         else:
-            out = forgetting_attention(q, k, v, log_fgate, head_first=w["head_first"], seq_start=seq_start)
+            out = forgetting_attention(q, k, v, log_fgate, head_first=w["head_first"], seq_start=seq_start,
+                                       adaptive_threshold=thr)
             out.backward(dout)
             q.grad = k.grad = v.grad = log_fgate.grad = None
 
@@ -639,7 +645,19 @@ def main():
     total = f_fwd if w["fwd_only"] else 3.5 * f_fwd  # bwd = 2.5 x fwd in the reference's convention
     value = total / sec * 1e-12
 
-    stages = stage_times(w, tensors, max(3, ns.steps))
+    stage_thr = thr
+    if thr == "auto":   # the (batch, head) thresholds the operator would derive, from the library's own kernel
+        from forgetting_transformer.ops import _lib
+        from forgetting_transformer.ops.forgetting_attention import _view
+        qh, kh = (x.detach().transpose(1, 2) if not w["head_first"] else x.detach() for x in (q, k))
+        stage_thr = torch.empty((w["B"], w["H"]), dtype=torch.float32, device="cuda")
+        scratch = torch.empty((w["B"], w["H"], 2), dtype=torch.int32, device="cuda")
+        dims = _lib.Dims(w["B"], w["H"], w["M"], w["N"], w["D"], _lib.DTYPE_BF16)
+        qv, kv = _view(qh), _view(kh)
+        _lib.check(_lib.load().fox_auto_threshold(C.byref(dims), C.byref(qv), C.byref(kv), 1.0 / math.sqrt(w["D"]),
+                                                  stage_thr.data_ptr(), scratch.data_ptr(),
+                                                  C.c_void_p(torch.cuda.current_stream().cuda_stream)), "fox_auto_threshold")
+    stages = stage_times(w, tensors, max(3, ns.steps), threshold=stage_thr)
     unit_flops = f_fwd / 2.0  # one causal matmul, B*H*T^2*D
     kern_flops = {"fwd": 2 * unit_flops, "bwd_dkdv": 4 * unit_flops, "bwd_dq": 3 * unit_flops}
     kernels = {}
@@ -649,12 +667,20 @@ def main():
             e["tflops"] = kern_flops[name] / t * 1e-12
             e["frac_of_peak"] = e["tflops"] / PEAK_BF16_TFLOPS
         kernels[name] = e
-    traffic, traffic_source = measured_traffic(ns.workload)
+    traffic, traffic_source = measured_traffic(ns.workload if thr is None else ns.workload + "_pruned")
     if w["fwd_only"]:  # few query rows against a long key sequence: one pass over K and V, HBM-bound
         dom = "fwd"
         pad = seq_start.float() if seq_start is not None else torch.zeros(w["B"], device="cuda")
         alg_bytes = ((2.0 * w["H"] * (w["N"] - pad) * w["D"] * 2).sum().item()
                      + 2 * w["B"] * w["H"] * w["M"] * w["D"] * 2 + w["B"] * w["H"] * w["N"] * 4)
+        gbps = alg_bytes / stages[dom] * 1e-9
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                    "frac": gbps / PEAK_HBM_GBPS, "traffic": traffic, "traffic_source": traffic_source,
+                    "algorithmic_bytes": alg_bytes, "avg_launch_ms": kernels[dom]["ms"]}
+    elif thr is not None:   # pruned step: every kernel is a stream over its inputs and outputs; dK/dV is the longest
+        dom = "bwd_dkdv"
+        S_, R_ = w["B"] * w["H"] * w["M"] * w["D"] * 2, w["B"] * w["H"] * w["M"] * 4
+        alg_bytes = 6 * S_ + 6 * R_   # q, k, v, do in; dk, dv out; lse, delta, row sums, c (rows and keys) in, dc out
         gbps = alg_bytes / stages[dom] * 1e-9
         roofline = {"kernel": dom, "bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                     "frac": gbps / PEAK_HBM_GBPS, "traffic": traffic, "traffic_source": traffic_source,
@@ -673,7 +699,8 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{ns.workload}: B{w['B']} M{w['M']} N{w['N']} H{w['H']} D{w['D']} bf16 "
                                f"{'fwd' if w['fwd_only'] else 'fwd+bwd'}, gate logits N({w['mean']},{w['std']}), "
-                               f"head_first={w['head_first']}, no pruning",
+                               f"head_first={w['head_first']}, "
+                               + ("no pruning" if thr is None else f"adaptive_threshold={thr}"),
                    "flops_convention": "fwd 2*B*H*T^2*D, bwd 5*B*H*T^2*D (causal)"},
         "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
         "roofline": roofline,
