@@ -212,7 +212,7 @@ def stage_times(w, tensors, iters, threshold=None):
     for name, fn in (("bwd_dq", lib.fox_attn_bwd_dq), ("bwd_dkdv", lib.fox_attn_bwd_dkdv)):
         out[name] = event_time(lambda fn=fn, name=name: _lib.check(fn(C.byref(bwd), stream), name), iters)
     out["cumsum_bwd"] = event_time(
-        lambda: _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg.data_ptr(), 0, 0, 0, B, H, N, stream), "cumsum_bwd"), iters)
+        lambda: _lib.check(lib.fox_cumsum_bwd(dc.data_ptr(), dg.data_ptr(), 0, 0, 0, None, B, H, N, stream), "cumsum_bwd"), iters)
     return out
 
 

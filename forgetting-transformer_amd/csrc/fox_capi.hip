@@ -319,22 +319,24 @@ int fox_gate_cumsum_fwd(const void* logits, int32_t logits_dtype, int64_t sb, in
 }
 
 int fox_gate_cumsum_bwd(const float* dc, const void* logits, int32_t logits_dtype, int64_t sb, int64_t sh, int64_t sn,
-                        void* dlogits, int64_t db, int64_t dh, int64_t dn, int32_t B, int32_t H, int32_t N, void* stream) {
+                        const int64_t* seq_start, void* dlogits, int64_t db, int64_t dh, int64_t dn, int32_t B, int32_t H,
+                        int32_t N, void* stream) {
   if (!dc || !logits || !dlogits) return fail(FOX_E_ARG, "dc, logits and dlogits must not be NULL");
   if (B <= 0 || H <= 0 || N <= 0) return fail(FOX_E_ARG, "B, H, N must be positive");
   if (logits_dtype < FOX_DTYPE_BF16 || logits_dtype > FOX_DTYPE_FP32) return fail(FOX_E_ARG, "logits_dtype must be FOX_DTYPE_BF16, FP16 or FP32 (got %d)", logits_dtype);
   if ((const void*)dc == dlogits || logits == dlogits) return fail(FOX_E_ARG, "dlogits must not alias dc or logits");
-  return check_hip(fox::launch_gate_cumsum_bwd(dc, logits, logits_dtype, sb, sh, sn, dlogits, db, dh, dn, B, H, N, (hipStream_t)stream),
+  return check_hip(fox::launch_gate_cumsum_bwd(dc, logits, logits_dtype, sb, sh, sn, seq_start, dlogits, db, dh, dn, B, H, N,
+                                               (hipStream_t)stream),
                    "fox_gate_cumsum_bwd");
 }
 
-int fox_cumsum_bwd(const float* dc, float* dg, int64_t dg_sb, int64_t dg_sh, int64_t dg_sn, int32_t B, int32_t H, int32_t N,
-                   void* stream) {
+int fox_cumsum_bwd(const float* dc, float* dg, int64_t dg_sb, int64_t dg_sh, int64_t dg_sn, const int64_t* seq_start, int32_t B,
+                   int32_t H, int32_t N, void* stream) {
   if (!dc || !dg) return fail(FOX_E_ARG, "dc and dg must not be NULL");
   if (B <= 0 || H <= 0 || N <= 0) return fail(FOX_E_ARG, "B, H, N must be positive");
   if (dc == dg) return fail(FOX_E_ARG, "dc and dg must not alias");
   if (dg_sb == 0 && dg_sh == 0 && dg_sn == 0) { dg_sb = (int64_t)H * N; dg_sh = N; dg_sn = 1; }   // contiguous (B,H,N)
-  return check_hip(fox::launch_cumsum_bwd(dc, dg, dg_sb, dg_sh, dg_sn, B, H, N, (hipStream_t)stream), "fox_cumsum_bwd");
+  return check_hip(fox::launch_cumsum_bwd(dc, dg, dg_sb, dg_sh, dg_sn, seq_start, B, H, N, (hipStream_t)stream), "fox_cumsum_bwd");
 }
 
 int fox_auto_threshold(const fox_dims* dims, const fox_view* q, const fox_view* k, float sm_scale, float* thr,
@@ -410,7 +412,7 @@ int fox_attn_bwd(const fox_bwd_args* args, void* stream) {
   FOX_TRY(fox_attn_bwd_dq(args, stream));
   FOX_TRY(fox_attn_bwd_dkdv(args, stream));
   return fox_cumsum_bwd(args->dlog_lambda, args->dlog_fgate, args->dlog_fgate_stride_b, args->dlog_fgate_stride_h,
-                        args->dlog_fgate_stride_n, args->dims.B, args->dims.H, args->dims.N, stream);
+                        args->dlog_fgate_stride_n, args->seq_start, args->dims.B, args->dims.H, args->dims.N, stream);
 }
 
 }  // extern "C"

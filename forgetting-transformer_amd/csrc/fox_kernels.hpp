@@ -99,8 +99,10 @@ hipError_t launch_cumsum_fwd(const float* g, int64_t sb, int64_t sh, int64_t sn,
 hipError_t launch_gate_cumsum_fwd(const void* logits, int dtype, int64_t sb, int64_t sh, int64_t sn, const int64_t* seq_start,
                                   float* log_fgate, float* c, int B, int H, int N, hipStream_t s);
 hipError_t launch_gate_cumsum_bwd(const float* dc, const void* logits, int dtype, int64_t sb, int64_t sh, int64_t sn,
-                                  void* dlogits, int64_t db, int64_t dh, int64_t dn, int B, int H, int N, hipStream_t s);
-hipError_t launch_cumsum_bwd(const float* dc, float* dg, int64_t db, int64_t dh, int64_t dn, int B, int H, int N, hipStream_t s);
+                                  const int64_t* seq_start, void* dlogits, int64_t db, int64_t dh, int64_t dn, int B, int H, int N,
+                                  hipStream_t s);
+hipError_t launch_cumsum_bwd(const float* dc, float* dg, int64_t db, int64_t dh, int64_t dn, const int64_t* seq_start, int B, int H,
+                             int N, hipStream_t s);
 hipError_t launch_auto_threshold(const View& q, const View& k, int B, int H, int M, int N, int D, int dtype, float sm_scale,
                                  float* thr, uint32_t* scratch, hipStream_t s);
 

@@ -98,13 +98,16 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(const float* __restr
   const float* src = in + b * sb + h * sh;
   float* dst = out + b * ob + h * oh;
   int seq = 0;
-  if (!REVERSE && seq_start) {
+  if (seq_start) {
     const int64_t s64 = seq_start[b];
     seq = (int)(s64 < 0 ? 0 : (s64 > N ? N : s64));
   }
+  // Reverse: the gradient of every gate up to and including position seq is the sum of all dc, zero in exact
+  // arithmetic (those gates shift every cumulative sum the kernels see by the same amount, or are zeroed by the
+  // forward); it is stored as an exact zero instead of the rounding noise of that sum.
   scan_row<REVERSE>(
       N, [&](int idx) { return (REVERSE || idx >= seq) ? src[(int64_t)idx * sn] : 0.f; },
-      [&](int idx, float sum) { dst[(int64_t)idx * on] = sum; });
+      [&](int idx, float sum) { dst[(int64_t)idx * on] = (REVERSE && idx <= seq) ? 0.f : sum; });
 }
 
 // Forget-gate logits in fp32, bf16 or fp16 (the output of the gate projection of the FoX layer).
@@ -165,18 +168,25 @@ __global__ __launch_bounds__(kScanThreads) void gate_scan_fwd_kernel(const void*
 // dtype and layout of the logits.
 template <int DT>
 __global__ __launch_bounds__(kScanThreads) void gate_scan_bwd_kernel(const float* __restrict__ dc, const void* __restrict__ logits,
-                                                            int64_t sb, int64_t sh, int64_t sn, void* __restrict__ dlogits,
-                                                            int64_t db, int64_t dh, int64_t dn, int H, int N) {
+                                                            int64_t sb, int64_t sh, int64_t sn, const int64_t* __restrict__ seq_start,
+                                                            void* __restrict__ dlogits, int64_t db, int64_t dh, int64_t dn, int H,
+                                                            int N) {
   const int bh = blockIdx.x, b = bh / H, h = bh % H;
   const float* src = dc + (int64_t)bh * N;
   const int64_t lbase = b * sb + h * sh, dbase = b * db + h * dh;
+  int seq = 0;
+  if (seq_start) {
+    const int64_t s64 = seq_start[b];
+    seq = (int)(s64 < 0 ? 0 : (s64 > N ? N : s64));
+  }
   scan_row<true>(
       N, [&](int idx) { return src[idx]; },
       [&](int idx, float sum) {
         const float x = load_logit<DT>(logits, lbase + (int64_t)idx * sn);
         const float z = __expf(-fabsf(x));
         const float r = __fdividef(z, 1.f + z);              // sigmoid(-|x|)
-        store_logit<DT>(dlogits, dbase + (int64_t)idx * dn, sum * (x < 0.f ? 1.f - r : r));
+        // positions up to and including seq: an exact zero, as in scan_kernel<true>
+        store_logit<DT>(dlogits, dbase + (int64_t)idx * dn, idx <= seq ? 0.f : sum * (x < 0.f ? 1.f - r : r));
       });
 }
 
@@ -193,12 +203,13 @@ hipError_t launch_gate_cumsum_fwd(const void* logits, int dtype, int64_t sb, int
 }
 
 hipError_t launch_gate_cumsum_bwd(const float* dc, const void* logits, int dtype, int64_t sb, int64_t sh, int64_t sn,
-                                  void* dlogits, int64_t db, int64_t dh, int64_t dn, int B, int H, int N, hipStream_t s) {
+                                  const int64_t* seq_start, void* dlogits, int64_t db, int64_t dh, int64_t dn, int B, int H, int N,
+                                  hipStream_t s) {
   const dim3 grid((unsigned)(B * H));
   switch (dtype) {
-    case 0: hipLaunchKernelGGL(gate_scan_bwd_kernel<0>, grid, dim3(kScanThreads), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
-    case 1: hipLaunchKernelGGL(gate_scan_bwd_kernel<1>, grid, dim3(kScanThreads), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
-    case 2: hipLaunchKernelGGL(gate_scan_bwd_kernel<2>, grid, dim3(kScanThreads), 0, s, dc, logits, sb, sh, sn, dlogits, db, dh, dn, H, N); break;
+    case 0: hipLaunchKernelGGL(gate_scan_bwd_kernel<0>, grid, dim3(kScanThreads), 0, s, dc, logits, sb, sh, sn, seq_start, dlogits, db, dh, dn, H, N); break;
+    case 1: hipLaunchKernelGGL(gate_scan_bwd_kernel<1>, grid, dim3(kScanThreads), 0, s, dc, logits, sb, sh, sn, seq_start, dlogits, db, dh, dn, H, N); break;
+    case 2: hipLaunchKernelGGL(gate_scan_bwd_kernel<2>, grid, dim3(kScanThreads), 0, s, dc, logits, sb, sh, sn, seq_start, dlogits, db, dh, dn, H, N); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
@@ -211,9 +222,10 @@ hipError_t launch_cumsum_fwd(const float* g, int64_t sb, int64_t sh, int64_t sn,
   return hipGetLastError();
 }
 
-hipError_t launch_cumsum_bwd(const float* dc, float* dg, int64_t db, int64_t dh, int64_t dn, int B, int H, int N, hipStream_t s) {
+hipError_t launch_cumsum_bwd(const float* dc, float* dg, int64_t db, int64_t dh, int64_t dn, const int64_t* seq_start, int B, int H,
+                             int N, hipStream_t s) {
   hipLaunchKernelGGL(scan_kernel<true>, dim3((unsigned)(B * H)), dim3(kScanThreads), 0, s, dc, (int64_t)H * N, (int64_t)N, (int64_t)1,
-                     (const int64_t*)nullptr, dg, db, dh, dn, H, N);
+                     seq_start, dg, db, dh, dn, H, N);
   return hipGetLastError();
 }
 

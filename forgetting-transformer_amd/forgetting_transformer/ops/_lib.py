@@ -107,11 +107,12 @@ SIGNATURES = {
     "fox_tile_config": (C.c_int, [C.c_int32] + [C.POINTER(C.c_int32)] * 4),
     "fox_cumsum_fwd": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                  C.c_int32, C.c_void_p]),
-    "fox_cumsum_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
+    "fox_cumsum_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
+                                 C.c_void_p]),
     "fox_gate_cumsum_fwd": (C.c_int, [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
-    "fox_gate_cumsum_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int64,
-                                      C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
+    "fox_gate_cumsum_bwd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p,
+                                      C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "fox_auto_threshold": (C.c_int, [C.POINTER(Dims), C.POINTER(View), C.POINTER(View), C.c_float, C.c_void_p, C.c_void_p,
                                      C.c_void_p]),
     "fox_attn_fwd": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),

@@ -342,7 +342,7 @@ def _backward(ctx, do):
             dgate = torch.empty_like(gate_logit)
             _lib.check(lib.fox_gate_cumsum_bwd(_ptr(dlog_lambda), _ptr(gate_logit), _GATE_DTYPES[gate_logit.dtype],
                                                gate_logit.stride(0), gate_logit.stride(1), gate_logit.stride(2),
-                                               _ptr(dgate), dgate.stride(0), dgate.stride(1), dgate.stride(2), B, H, N,
+                                               _ptr(seq_start), _ptr(dgate), dgate.stride(0), dgate.stride(1), dgate.stride(2), B, H, N,
                                                stream), "fox_gate_cumsum_bwd")
     return dq, dk, dv, dgate
 

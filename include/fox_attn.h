@@ -80,9 +80,11 @@ int fox_cumsum_fwd(const float* g, int64_t g_sb, int64_t g_sh, int64_t g_sn, con
  * dg[b,h,l] = sum_{n>=l} dc[b,h,n]; dc is (B,H,N) contiguous fp32, dg is fp32 with element strides
  * (dg_sb, dg_sh, dg_sn) -- the layout of the caller's log_fgate, so that autograd can take the gradient as it
  * is -- or (B,H,N) contiguous when all three strides are 0.  Replaces the reverse cumulative sum at :390-392.
+ * Positions l <= seq_start[b] (l = 0 when seq_start is NULL) get an exact 0: their gradient is the sum of all dc,
+ * which vanishes in exact arithmetic (the reference returns the rounding noise of that sum).
  */
-int fox_cumsum_bwd(const float* dc, float* dg, int64_t dg_sb, int64_t dg_sh, int64_t dg_sn, int32_t B, int32_t H,
-                   int32_t N, void* stream);
+int fox_cumsum_bwd(const float* dc, float* dg, int64_t dg_sb, int64_t dg_sh, int64_t dg_sn, const int64_t* seq_start,
+                   int32_t B, int32_t H, int32_t N, void* stream);
 
 /*
  * The prologue of the FoX layer fused with the scan: c[b,h,n] = sum_{seq_start[b] <= l <= n} logsigmoid(x[b,h,l])
@@ -98,9 +100,11 @@ int fox_gate_cumsum_fwd(const void* logits, int32_t logits_dtype, int64_t sb, in
 /*
  * dlogits[b,h,l] = (sum_{n>=l} dc[b,h,n]) * (1 - sigmoid(x[b,h,l])): the reverse cumulative sum (:390-392)
  * fused with the derivative of logsigmoid; dlogits has the dtype of the logits and its own element strides.
+ * Positions l <= seq_start[b] (l = 0 when seq_start is NULL) get an exact 0, as in fox_cumsum_bwd.
  */
 int fox_gate_cumsum_bwd(const float* dc, const void* logits, int32_t logits_dtype, int64_t sb, int64_t sh, int64_t sn,
-                        void* dlogits, int64_t db, int64_t dh, int64_t dn, int32_t B, int32_t H, int32_t N, void* stream);
+                        const int64_t* seq_start, void* dlogits, int64_t db, int64_t dh, int64_t dn, int32_t B, int32_t H,
+                        int32_t N, void* stream);
 
 /*
  * thr[b,h] = -(2 * max_m|q| * max_n|k| * sm_scale + log N) - 10, with the row norms
