@@ -213,12 +213,15 @@ int make_norm_gate(const fox_norm_gate_args* a, fox::NormGateK& k, bool bwd) {
 
 // The forward with its key-split scratch passed separately: the caller's workspace (fox_attn_fwd) or the
 // library's own array (fox_attn_fwd_noalloc).  workspace == NULL never splits keys.
-int fwd_impl(const fox_fwd_args* args, void* workspace, int64_t workspace_bytes, void* stream, const char* what) {
+// epi: the norm-and-gate epilogue (already validated), or NULL.  With an epilogue, shapes the unsplit kernel does
+// not handle run the plain forward followed by the standalone norm kernel.
+int fwd_impl(const fox_fwd_args* args, void* workspace, int64_t workspace_bytes, void* stream, const char* what,
+             const fox_fwd_epilogue* epi = nullptr) {
   FOX_TRY(check_dims(&args->dims));
   FOX_TRY(check_view(&args->q, "q"));
   FOX_TRY(check_view(&args->k, "k"));
   FOX_TRY(check_view(&args->v, "v"));
-  FOX_TRY(check_view(&args->o, "o"));
+  if (!(epi && !args->o.ptr)) FOX_TRY(check_view(&args->o, "o"));
   FOX_TRY(check_extent(&args->k, args->dims.N, args->dims.D, "k"));
   FOX_TRY(check_extent(&args->v, args->dims.N, args->dims.D, "v"));
   if (!args->log_lambda || !args->lse) return fail(FOX_E_ARG, "log_lambda and lse must not be NULL");
@@ -247,6 +250,32 @@ int fwd_impl(const fox_fwd_args* args, void* workspace, int64_t workspace_bytes,
       k.ws_ml = k.ws_o + (int64_t)k.splits * k.B * k.H * k.M * args->dims.D;
     }
   }
+  if (epi) {
+    const int D = args->dims.D;
+    if (k.M == 1 || k.splits > 1) {
+      // two passes: the plain forward, then the norm over o as (B*M rows, H heads)
+      const fox_view* vs[3] = {&args->o, &epi->y, &epi->gate};
+      for (int i = 0; i < 3; ++i) {
+        if (i == 2 && epi->activation == FOX_ACT_NONE) break;
+        if (!vs[i]->ptr || vs[i]->stride_h != D || vs[i]->stride_b != (int64_t)k.M * vs[i]->stride_t)
+          return fail(FOX_E_ARG, "%s: a key-split or single-query shape needs o, gate and y with adjacent heads "
+                                 "(stride_h == D, stride_b == M * stride_t)", what);
+      }
+      FOX_TRY(check_hip(fox::launch_fwd(k, D, args->dims.dtype, (hipStream_t)stream), what));
+      fox::NormGateK n{};
+      n.x = (const uint16_t*)args->o.ptr; n.x_sr = args->o.stride_t;
+      n.g = epi->activation == FOX_ACT_NONE ? nullptr : (const uint16_t*)epi->gate.ptr; n.g_sr = epi->gate.stride_t;
+      n.y = (uint16_t*)epi->y.ptr; n.y_sr = epi->y.stride_t;
+      n.w = epi->weight; n.rstd = epi->rstd; n.R = (int64_t)k.B * k.M; n.G = k.H; n.eps = epi->eps;
+      return check_hip(fox::launch_norm_gate(n, D, args->dims.dtype, false, epi->activation, (hipStream_t)stream), what);
+    }
+    k.epi.gate = epi->activation == FOX_ACT_NONE ? fox::View{} : to_view(epi->gate);
+    k.epi.y = to_view(epi->y);
+    k.epi.w = epi->weight;
+    k.epi.rstd = epi->rstd;
+    k.epi.eps = epi->eps;
+    k.epi.act = epi->activation;
+  }
   return check_hip(fox::launch_fwd(k, args->dims.D, args->dims.dtype, (hipStream_t)stream), what);
 }
 
@@ -267,6 +296,18 @@ int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_b
   if (kv_block_n) *kv_block_n = fox::kKvBN;
   if (kv_block_m) *kv_block_m = fox::kKvBM;
   return FOX_OK;
+}
+
+int fox_attn_fwd_norm_gate(const fox_fwd_args* args, const fox_fwd_epilogue* epi, void* stream) {
+  if (!args || !epi) return fail(FOX_E_ARG, "args and epilogue must not be NULL");
+  if (epi->activation != FOX_ACT_SIGMOID && epi->activation != FOX_ACT_SWISH && epi->activation != FOX_ACT_NONE)
+    return fail(FOX_E_ARG, "activation must be FOX_ACT_SIGMOID, FOX_ACT_SWISH or FOX_ACT_NONE (got %d)", epi->activation);
+  FOX_TRY(check_view(&epi->y, "y"));
+  if (epi->activation != FOX_ACT_NONE) FOX_TRY(check_view(&epi->gate, "gate"));
+  if (!epi->weight || !epi->rstd) return fail(FOX_E_ARG, "weight and rstd must not be NULL");
+  if (((uintptr_t)epi->weight & 15) != 0) return fail(FOX_E_ALIGN, "weight must be 16-byte aligned");
+  if (epi->y.ptr == args->o.ptr) return fail(FOX_E_ARG, "y must not alias o");
+  return fwd_impl(args, args->workspace, args->workspace_bytes, stream, "fox_attn_fwd_norm_gate", epi);
 }
 
 int fox_norm_gate_fwd(const fox_norm_gate_args* args, void* stream) {

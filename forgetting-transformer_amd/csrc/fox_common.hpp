@@ -302,6 +302,77 @@ __device__ __forceinline__ void store_rows_via_lds(char* stage, const f32x16 (&a
   __builtin_amdgcn_wave_barrier();   // the staging area may be rewritten after this
 }
 
+// Gate activations of the per-head RMS norm (FOX_ACT_* of the public header).
+enum : int { kActSigmoid = 0, kActSwish = 1, kActNone = 2 };
+__device__ __forceinline__ float sigmoidf(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// store_rows_via_lds with the gated per-head RMS norm applied on the way out: besides the rows themselves
+// (x = acc * mul rounded to 16 bits, to x_dst unless that is null) it writes
+//   y[row, :] = x * rstd[row] * w[:] * act(gate[row, :]),   rstd = 1 / sqrt(mean_d x^2 + eps),
+// computed from the rounded x, as a separate normalisation pass over the stored rows would, and rstd itself
+// (one float per row, rstd_stride apart).  gate is not read when act is kActNone.  The 16 spare bytes that
+// pad every staged row carry its rstd from the lanes that own the row to the lanes that store it.  Nothing of
+// the epilogue is prefetched while the accumulators are live: the kernels that end with it run at the register
+// limit of their occupancy.
+template <typename Tr, int D>
+__device__ __forceinline__ void store_rows_norm_gate(char* stage, const f32x16 (&acc)[(D + 31) / 32], float mul, uint16_t* x_dst,
+                                                     int64_t x_stride, const uint16_t* gate, int64_t gate_stride, uint16_t* y_dst,
+                                                     int64_t y_stride, const float* w, float* rstd_dst, int64_t rstd_stride,
+                                                     float eps, int act, int row0, int row_limit, int lane) {
+  constexpr int DB = (D + 31) / 32, CH = D / 8, RS = 2 * D + 16, NIT = (32 * CH + kWave - 1) / kWave;
+  const int g = lane >> 5, i = lane & 31;
+  float ss = 0.f;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const int d = 32 * db + 8 * q4 + 4 * g;
+      if (d < D) {
+        u32x2 v;
+        v[0] = Tr::pack2(acc[db][4 * q4 + 0] * mul, acc[db][4 * q4 + 1] * mul);
+        v[1] = Tr::pack2(acc[db][4 * q4 + 2] * mul, acc[db][4 * q4 + 3] * mul);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) ss += Tr::lo(v[e]) * Tr::lo(v[e]) + Tr::hi(v[e]) * Tr::hi(v[e]);
+        *reinterpret_cast<u32x2*>(stage + i * RS + 2 * d) = v;
+      }
+    }
+  ss = half_sum(ss);  // the two halves of the wave hold the two halves of every row
+  const float rs_own = 1.0f / sqrtf(ss / D + eps);
+  if (g == 0) *reinterpret_cast<float*>(stage + i * RS + 2 * D) = rs_own;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int idx = it * kWave + lane, row = idx / CH, ch = idx % CH;
+    if ((32 * CH % kWave == 0 || idx < 32 * CH) && row0 + row < row_limit) {
+      u32x4 gv = {0u, 0u, 0u, 0u};
+      if (act != kActNone) gv = *reinterpret_cast<const u32x4*>(gate + (int64_t)(row0 + row) * gate_stride + 8 * ch);
+      const u32x4 xv = *reinterpret_cast<const u32x4*>(stage + row * RS + 16 * ch);
+      const float rs = *reinterpret_cast<const float*>(stage + row * RS + 2 * D);
+      if (x_dst) *reinterpret_cast<u32x4*>(x_dst + (int64_t)(row0 + row) * x_stride + 8 * ch) = xv;
+      const f32x4 w0 = *reinterpret_cast<const f32x4*>(w + 8 * ch), w1 = *reinterpret_cast<const f32x4*>(w + 8 * ch + 4);
+      u32x4 yv;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float y0 = Tr::lo(xv[e]) * rs * (e < 2 ? w0[2 * e] : w1[2 * e - 4]);
+        float y1 = Tr::hi(xv[e]) * rs * (e < 2 ? w0[2 * e + 1] : w1[2 * e - 3]);
+        if (act != kActNone) {
+          const float g0 = Tr::lo(gv[e]), g1 = Tr::hi(gv[e]);
+          const float s0 = sigmoidf(g0), s1 = sigmoidf(g1);
+          y0 *= act == kActSwish ? g0 * s0 : s0;
+          y1 *= act == kActSwish ? g1 * s1 : s1;
+        }
+        yv[e] = Tr::pack2(y0, y1);
+      }
+      *reinterpret_cast<u32x4*>(y_dst + (int64_t)(row0 + row) * y_stride + 8 * ch) = yv;
+      if (ch == 0) rstd_dst[(int64_t)(row0 + row) * rstd_stride] = rs;
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();   // the staging area may be rewritten after this
+}
+
 // Start value of a 32x32 MFMA accumulator whose row r carries the per-row term
 // t[row0 + r] (read from LDS): the matrix pipe then adds the dot products to it for
 // free, which saves one vector instruction per score.

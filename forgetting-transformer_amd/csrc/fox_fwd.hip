@@ -25,6 +25,8 @@
 // stored log-normaliser.  Columns left of seq_start (and beyond N) get
 // (c_n - c_ref) = +inf, which makes x = -inf without a compare in the loop; only
 // tiles crossing the diagonal run the causal compare (separate code path).
+#include <stddef.h>
+
 #include "fox_common.hpp"
 #include "fox_kernels.hpp"
 
@@ -231,8 +233,11 @@ struct TileDma {
   }
 };
 
-template <typename Tr, int D, bool SPLIT>
+// EPI: the variant whose epilogue also applies the layer's output norm and gate (a.epi); a variant of its own so
+// that the plain kernel's register allocation is not touched by it.
+template <typename Tr, int D, bool SPLIT, bool EPI = false>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
+  static_assert(!(SPLIT && EPI), "partial results of a key split are not normalised");
   constexpr int BM = kFwdBM, BN = kFwdBN;
   constexpr int KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
   static_assert(BM == 128, "four waves of 32 rows");
@@ -454,7 +459,21 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
   wait_vmem_all();  // whatever was requested last (possibly an empty tile) has landed
   __syncthreads();  // every wave is done with the last tile
   char* stage = wave == 0 ? k_tile0 : wave == 1 ? k_tile1 : wave == 2 ? v_tile0 : v_tile1;
-  store_rows_via_lds<Tr, D>(stage, oacc, inv, op, a.o.st, m0 + 32 * wave, M, lane);
+  if constexpr (EPI) {  // the layer's output norm and gate, applied while the rows are on their way out
+    // The epilogue's arguments are fetched from the kernel argument block only here, through a pointer the
+    // compiler cannot see through: loaded at kernel entry they would occupy scalar registers across the key loop.
+    typedef const char __attribute__((address_space(4)))* kernarg_bytes;
+    typedef const FwdEpilogue __attribute__((address_space(4)))* kernarg_epilogue;
+    kernarg_epilogue ep = (kernarg_epilogue)((kernarg_bytes)__builtin_amdgcn_kernarg_segment_ptr() + offsetof(FwdK, epi));
+    asm volatile("" : "+s"(ep));
+    const uint16_t* gp = ep->gate.ptr ? ep->gate.ptr + b * ep->gate.sb + h * ep->gate.sh : nullptr;
+    uint16_t* yp = const_cast<uint16_t*>(ep->y.ptr) + b * ep->y.sb + h * ep->y.sh;
+    store_rows_norm_gate<Tr, D>(stage, oacc, inv, a.o.ptr ? op : nullptr, a.o.st, gp, ep->gate.st, yp, ep->y.st,
+                                ep->w + h * D, ep->rstd + (int64_t)b * M * a.H + h, a.H, ep->eps, ep->act, m0 + 32 * wave,
+                                M, lane);
+  } else {
+    store_rows_via_lds<Tr, D>(stage, oacc, inv, op, a.o.st, m0 + 32 * wave, M, lane);
+  }
 }
 
 // Merge the partial results of the key splits of one query row:
@@ -500,6 +519,10 @@ __global__ __launch_bounds__(256) void combine_kernel(const FwdK a) {
   template __global__ void fwd_kernel<TR, 32, false>(const FwdK);        \
   template __global__ void fwd_kernel<TR, 64, false>(const FwdK);        \
   template __global__ void fwd_kernel<TR, 128, false>(const FwdK);       \
+  template __global__ void fwd_kernel<TR, 16, false, true>(const FwdK);  \
+  template __global__ void fwd_kernel<TR, 32, false, true>(const FwdK);  \
+  template __global__ void fwd_kernel<TR, 64, false, true>(const FwdK);  \
+  template __global__ void fwd_kernel<TR, 128, false, true>(const FwdK); \
   template __global__ void fwd_kernel<TR, 16, true>(const FwdK);         \
   template __global__ void fwd_kernel<TR, 32, true>(const FwdK);         \
   template __global__ void fwd_kernel<TR, 64, true>(const FwdK);         \
@@ -513,11 +536,14 @@ FOX_INSTANTIATE_FWD(Fp16)
 
 template <typename Tr, int D>
 static hipError_t launch_fwd_d(const FwdK& a, int dtype, hipStream_t s) {
+  if (a.epi.y.ptr && (a.M == 1 || a.splits > 1)) return hipErrorInvalidValue;  // the epilogue lives in the unsplit kernel only
   if (a.M == 1) {  // decode step: the streaming kernel, one workgroup per (batch, head, key split)
     const hipError_t e = launch_fwd_decode(a, D, dtype, s);
     if (e != hipSuccess || a.splits <= 1) return e;
   } else if (a.splits <= 1) {
-    hipLaunchKernelGGL((fwd_kernel<Tr, D, false>), dim3((unsigned)(a.n_mtiles * a.B * a.H)), dim3(256), 0, s, a);
+    const dim3 grid((unsigned)(a.n_mtiles * a.B * a.H));
+    if (a.epi.y.ptr) hipLaunchKernelGGL((fwd_kernel<Tr, D, false, true>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((fwd_kernel<Tr, D, false>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
   } else {
     hipLaunchKernelGGL((fwd_kernel<Tr, D, true>), dim3((unsigned)(a.n_mtiles * a.splits * a.B * a.H)), dim3(256), 0, s, a);

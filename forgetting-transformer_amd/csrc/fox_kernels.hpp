@@ -11,6 +11,16 @@ struct View {
   int64_t sb, sh, st;
 };
 
+// Optional epilogue of the forward: the gated per-head RMS norm of the output rows (see store_rows_norm_gate).
+// Off when y.ptr is null.  gate and y are (B, H, M, D) views like o; w is (H*D) fp32; rstd is (B, M, H) fp32.
+struct FwdEpilogue {
+  View gate, y;
+  const float* w;
+  float* rstd;
+  float eps;
+  int act;
+};
+
 struct FwdK {
   View q, k, v, o;
   const float* c;
@@ -24,6 +34,7 @@ struct FwdK {
   int splits;      // key splits of the forward (1 = none)
   float* ws_o;     // (splits, B, H, M, D) partial accumulators
   float* ws_ml;    // (splits, B, H, M, 2) partial row maximum and row sum
+  FwdEpilogue epi; // only for splits == 1 and M > 1 (the launcher rejects it otherwise)
 };
 
 struct BwdK {

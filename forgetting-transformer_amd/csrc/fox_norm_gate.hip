@@ -36,10 +36,6 @@ __device__ __forceinline__ u32x4 pack8v(const float (&f)[8]) {
   for (int e = 0; e < 4; ++e) r[e] = Tr::pack2(f[2 * e], f[2 * e + 1]);
   return r;
 }
-__device__ __forceinline__ float sigmoidf(float x) { return 1.0f / (1.0f + __expf(-x)); }
-
-enum : int { kActSigmoid = 0, kActSwish = 1, kActNone = 2 };  // FOX_ACT_* of the public header
-
 template <typename Tr, int D, int ACT>
 __global__ __launch_bounds__(256) void norm_gate_fwd_kernel(const NormGateK a) {
   constexpr int CH = D / 8;

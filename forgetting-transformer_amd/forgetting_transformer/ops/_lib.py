@@ -99,6 +99,16 @@ class NormGateArgs(C.Structure):
     ]
 
 
+class FwdEpilogue(C.Structure):
+    _fields_ = [
+        ("gate", View), ("y", View),
+        ("weight", C.c_void_p),
+        ("rstd", C.c_void_p),
+        ("eps", C.c_float),
+        ("activation", C.c_int32),
+    ]
+
+
 # every symbol include/fox_attn.h declares: name -> (restype, argtypes)
 SIGNATURES = {
     "fox_version": (C.c_int, []),
@@ -117,6 +127,7 @@ SIGNATURES = {
                                      C.c_void_p]),
     "fox_attn_fwd": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),
     "fox_attn_fwd_noalloc": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),
+    "fox_attn_fwd_norm_gate": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(FwdEpilogue), C.c_void_p]),
     "fox_attn_fwd_workspace_bytes": (C.c_int, [C.POINTER(Dims), C.POINTER(C.c_int64)]),
     "fox_attn_bwd_delta": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),
     "fox_attn_bwd_dkdv": (C.c_int, [C.POINTER(BwdArgs), C.c_void_p]),

@@ -22,8 +22,8 @@ import torch
 
 from . import _lib
 
-__all__ = ["forgetting_attention", "forgetting_attention_from_logits", "qk_norm_threshold", "ForgettingAttention",
-           "ForgettingAttentionFromLogits"]
+__all__ = ["forgetting_attention", "forgetting_attention_from_logits", "forgetting_attention_norm_gate",
+           "qk_norm_threshold", "ForgettingAttention", "ForgettingAttentionFromLogits", "ForgettingAttentionNormGate"]
 
 _DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
 
@@ -162,6 +162,65 @@ class ForgettingAttentionFromLogits(torch.autograd.Function):
         return _backward(ctx, do) + (None,) * 3
 
 
+class ForgettingAttentionNormGate(torch.autograd.Function):
+    """The operator followed by the layer's per-head RMS norm and output gate
+    (``modeling_forgetting_transformer.py:417-422``), with that norm applied in the epilogue of the
+    forward kernel: the attention output is normalised while it leaves the kernel instead of being
+    read back by a kernel of its own.  The backward runs the norm's backward kernel on ``dy`` and
+    feeds its ``dx`` to the operator's backward.  ``gate`` is None for the ungated norm."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, log_fgate, gate, weight, seq_start, sm_scale, adaptive_threshold, activation, eps,
+                fgate_is_logit=False):
+        B, H, M, D = q.shape
+        assert weight.shape == (H * D,), "weight must have shape (heads * head_dim,)"
+        if gate is not None:
+            assert gate.shape == q.shape, "gate must have the shape of q"
+            assert gate.dtype == q.dtype, "gate must have the dtype of q"
+            gate = _heads_adjacent(gate)
+        w32 = weight.detach().float().contiguous()
+        y = _forward(ctx, fgate_is_logit, q, k, v, log_fgate, seq_start, True, sm_scale, adaptive_threshold, False, False,
+                     epilogue=(gate, w32, activation, float(eps)))
+        ctx.norm_meta = (activation, float(eps), weight.dtype, gate is not None)
+        if fgate_is_logit:  # the fp32 log gates are a by-product of the fused scan (see ForgettingAttentionFromLogits)
+            ctx.mark_non_differentiable(ctx.log_fgate)
+            return y, ctx.log_fgate
+        return y
+
+    @staticmethod
+    def backward(ctx, dy, *ignored):
+        q, o = ctx.saved_tensors[0], ctx.saved_tensors[3]
+        gate, w32, rstd = ctx.saved_tensors[9:12]
+        act, eps, w_dtype, gated = ctx.norm_meta
+        B, H, M, D = q.shape
+        rows, width = B * M, H * D
+        lib = _lib.load()
+        dy = _heads_adjacent(dy)
+        do = torch.empty((B, M, H, D), dtype=q.dtype, device=q.device).transpose(1, 2)
+        dgate = torch.empty((B, M, H, D), dtype=q.dtype, device=q.device).transpose(1, 2) if gated else None
+        dw = torch.empty((width,), dtype=torch.float32, device=q.device)
+        ws_bytes = C.c_int64(0)
+        _lib.check(lib.fox_norm_gate_workspace_bytes(rows, H, D, C.byref(ws_bytes)), "fox_norm_gate_workspace_bytes")
+        ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q.device)
+        args = _lib.NormGateArgs(rows, H, D, _DTYPES[q.dtype], act, eps, o.data_ptr(), o.stride(2),
+                                 gate.data_ptr() if gated else None, gate.stride(2) if gated else 0,
+                                 w32.data_ptr(), None, 0, rstd.data_ptr(), dy.data_ptr(), dy.stride(2),
+                                 do.data_ptr(), do.stride(2), dgate.data_ptr() if gated else None,
+                                 dgate.stride(2) if gated else 0, dw.data_ptr(), ws.data_ptr())
+        with _on_device(q.device):
+            _lib.check(lib.fox_norm_gate_bwd(C.byref(args), _stream(q.device)), "fox_norm_gate_bwd")
+        dq, dk, dv, dlog_fgate = _backward(ctx, do)
+        return dq, dk, dv, dlog_fgate, dgate, dw.to(w_dtype), None, None, None, None, None, None
+
+
+def _heads_adjacent(x: torch.Tensor) -> torch.Tensor:
+    """(B, H, M, D) tensor whose memory is (B, M, H, D) contiguous, 16-byte aligned: one row of heads * head_dim
+    elements per token, the layout of the layer's (batch, time, hidden) tensors.  Copies only when needed."""
+    B, H, M, D = x.shape
+    ok = x.stride() == (M * H * D, D, H * D, 1) and x.data_ptr() % 16 == 0
+    return x if ok else x.transpose(1, 2).contiguous().transpose(1, 2)
+
+
 _GATE_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16, torch.float32: _lib.DTYPE_FP32}
 
 
@@ -182,7 +241,7 @@ def _constant_threshold(value, B, H, device):
 
 
 def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
-             return_log_normalizer, return_start_index):
+             return_log_normalizer, return_start_index, epilogue=None):
     assert causal, "Only causal attention is supported"
     Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
     assert Dq == Dk == Dv, "feature size of q, k, v should be equal"
@@ -277,7 +336,13 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
                                           log_fgate.stride(2), _ptr(seq_start), _ptr(log_lambda), B, H, N, stream),
                        "fox_cumsum_fwd")
 
-        o = torch.empty_like(q)
+        y = rstd = None
+        if epilogue is None:
+            o = torch.empty_like(q)
+        else:  # o and y as rows of heads * head_dim per token: what the norm's backward and the output projection read
+            o = torch.empty((B, M, H, D), dtype=q.dtype, device=device).transpose(1, 2)
+            y = torch.empty((B, M, H, D), dtype=q.dtype, device=device).transpose(1, 2)
+            rstd = torch.empty((B, M, H), dtype=torch.float32, device=device)
         first_block = None
         if return_start_index:
             block_m, _, _, _ = _lib.tile_config(D)
@@ -287,10 +352,18 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
                             None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
                             sm_scale, None if first_block is None else first_block.data_ptr(),
                             None if workspace is None else workspace.data_ptr(), ws_bytes)
-        _lib.check(lib.fox_attn_fwd(C.byref(args), stream), "fox_attn_fwd")
+        if epilogue is None:
+            _lib.check(lib.fox_attn_fwd(C.byref(args), stream), "fox_attn_fwd")
+        else:
+            gate, w32, act, eps = epilogue
+            epi = _lib.FwdEpilogue(_view(gate) if gate is not None else _lib.View(), _view(y), w32.data_ptr(),
+                                   rstd.data_ptr(), eps, act)
+            _lib.check(lib.fox_attn_fwd_norm_gate(C.byref(args), C.byref(epi), stream), "fox_attn_fwd_norm_gate")
 
-    ctx.save_for_backward(q, k, v, o, L, log_lambda, seq_start, adaptive_threshold,
-                          log_fgate if gate_is_logit else None)
+    saved = (q, k, v, o, L, log_lambda, seq_start, adaptive_threshold, log_fgate if gate_is_logit else None)
+    if epilogue is not None:
+        saved += (epilogue[0], epilogue[1], rstd)
+    ctx.save_for_backward(*saved)
     ctx.sm_scale = sm_scale
     ctx.causal = causal
     ctx.has_seq_start = has_seq_start
@@ -304,10 +377,11 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
         outs = (o, L if return_log_normalizer else None, start_index)
         ctx.mark_non_differentiable(*[t for t in outs[1:] if t is not None])
         return outs
-    return o
+    return o if epilogue is None else y
+
 
 def _backward(ctx, do):
-    q, k, v, o, L, log_lambda, seq_start, adaptive_threshold, gate_logit = ctx.saved_tensors
+    q, k, v, o, L, log_lambda, seq_start, adaptive_threshold, gate_logit = ctx.saved_tensors[:9]
     B, H, M, D = q.shape
     N = k.shape[2]
     device = q.device
@@ -426,6 +500,57 @@ def forgetting_attention_from_logits(
     if not head_first:
         out, log_fgate = out.transpose(1, 2), log_fgate.transpose(1, 2)
     return out, log_fgate
+
+
+_NORM_ACTS = {"sigmoid": _lib.ACT_SIGMOID, "swish": _lib.ACT_SWISH, "silu": _lib.ACT_SWISH}
+
+
+def forgetting_attention_norm_gate(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    log_fgate: torch.Tensor,
+    gate: Optional[torch.Tensor],
+    norm_weight: torch.Tensor,
+    *,
+    activation: str = "sigmoid",
+    eps: float = 1e-6,
+    head_first: bool = False,
+    seq_start: Optional[torch.Tensor] = None,
+    sm_scale: Optional[float] = None,
+    adaptive_threshold: Optional[Union[Literal["auto"], float, torch.Tensor]] = None,
+    fgate_is_logit: bool = False,
+):
+    """``group_norm_gated(forgetting_attention(q, k, v, log_fgate, ...), gate, norm_weight, is_rms_norm=True,
+    num_groups=heads)`` in one forward kernel: what the FoX layer computes between the attention and its output
+    projection (``modeling_forgetting_transformer.py:396-422``).
+
+    ``gate`` has the shape and dtype of q (the layer's ``ogate_proj(hidden_states)`` viewed per head), or is None
+    for the ungated output norm (``:245, :422``); ``norm_weight`` is ``(heads * head_dim,)``; every other argument
+    is as in ``forgetting_attention``.  Returns the normalised, gated output in the shape of q; with
+    head_first=False it is contiguous, so ``.reshape(batch, seqlen, heads * head_dim)`` is a view.  Gradients
+    flow to q, k, v, log_fgate, gate and norm_weight.
+
+    With ``fgate_is_logit=True`` the fourth argument is the gate *logits* (bfloat16, float16 or float32) as in
+    ``forgetting_attention_from_logits`` and the result is ``(y, log_fgate)``: the whole chain from the layer's
+    gate projection to the input of its output projection in one scan kernel and one attention kernel.
+    """
+    for name, entry in dict(q=q, k=k, v=v).items():
+        assert entry.dtype in [torch.float16, torch.bfloat16], (
+            f"Only torch.float16 or torch.bfloat16 are supported for q/k/v, but got {entry.dtype} for {name}.")
+    if gate is not None and activation not in _NORM_ACTS:
+        raise ValueError(f"Unsupported activation: {activation}")
+    if not head_first:
+        q, k, v = [item.transpose(1, 2) for item in (q, k, v)]
+        log_fgate = log_fgate.transpose(1, 2)
+        gate = gate.transpose(1, 2) if gate is not None else None
+    act = _NORM_ACTS[activation] if gate is not None else _lib.ACT_NONE
+    out = ForgettingAttentionNormGate.apply(q, k, v, log_fgate, gate, norm_weight, seq_start, sm_scale,
+                                            adaptive_threshold, act, eps, fgate_is_logit)
+    if fgate_is_logit:
+        y, lg = out
+        return (y, lg) if head_first else (y.transpose(1, 2), lg.transpose(1, 2))
+    return out if head_first else out.transpose(1, 2)
 
 
 @torch.no_grad()

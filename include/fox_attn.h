@@ -280,6 +280,31 @@ int fox_norm_gate_bwd(const fox_norm_gate_args* args, void* stream);
 /* Size of the backward's workspace for `rows` rows of G heads of D elements. */
 int fox_norm_gate_workspace_bytes(int64_t rows, int32_t G, int32_t D, int64_t* bytes);
 
+/*
+ * The forward with the layer's output norm and gate applied in its epilogue: while a query tile's output rows
+ * are on their way from the accumulators to memory, the kernel also writes
+ *   y[b,h,m,:] = o[b,h,m,:] * rstd[b,m,h] * weight[h,:] * act(gate[b,h,m,:]),  rstd = 1/sqrt(mean_d o^2 + eps),
+ * computed from the rounded 16-bit o, i.e. what fox_attn_fwd followed by fox_norm_gate_fwd over o gives, without
+ * the second pass over o.  Fuses forgetting_attention (ops/forgetting_attention.py:505-693) with the call of
+ * FusedGroupNormGated / GroupNorm on its output (modeling_forgetting_transformer.py:243-245, :417-422;
+ * fuse_norm_gate.py:132-206).  gate and y are (B,H,M,D) views like o (gate may be NULL with FOX_ACT_NONE);
+ * weight is (H*D) fp32; rstd is (B,M,H) fp32 contiguous: the layout fox_norm_gate_bwd reads with rows = (b,m)
+ * and G = H.  args->o may have a NULL ptr when the caller needs only y (inference), except for the shapes below.
+ * Shapes whose forward splits the key loop (fox_attn_fwd_workspace_bytes() > 0 with a workspace given) and
+ * M == 1 run fox_attn_fwd and then the standalone norm kernel; that needs o, and o, gate and y with adjacent
+ * heads (stride_h == D, stride_b == M * stride_t), otherwise FOX_E_ARG.
+ */
+typedef struct fox_fwd_epilogue {
+  fox_view gate;        /* read; 16-bit, same dtype as q */
+  fox_view y;           /* written */
+  const float* weight;
+  float* rstd;          /* written */
+  float eps;
+  int32_t activation;   /* FOX_ACT_* */
+} fox_fwd_epilogue;
+
+int fox_attn_fwd_norm_gate(const fox_fwd_args* args, const fox_fwd_epilogue* epilogue, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

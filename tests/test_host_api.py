@@ -250,6 +250,37 @@ def test_no_cpu_fallback():
         forgetting_attention(q, k, v, g, head_first=True, adaptive_threshold=-10.0, seq_start=torch.zeros(2, dtype=torch.long))
 
 
+def test_norm_gate_epilogue_wrapper_checks():
+    """forgetting_attention_norm_gate validates on the host before any launch, has no CPU path, and the C entry point
+    rejects a bad epilogue without touching the device."""
+    from forgetting_transformer import forgetting_attention_norm_gate
+    q, k, v, g = _cpu_inputs()
+    B, T, H, D = q.shape
+    gate, w = torch.zeros_like(q), torch.ones(H * D)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        forgetting_attention_norm_gate(q, k, v, g, gate, w)
+    with pytest.raises(AssertionError, match="weight must have shape"):
+        forgetting_attention_norm_gate(q, k, v, g, gate, w[:-1])
+    with pytest.raises(AssertionError, match="shape of q"):
+        forgetting_attention_norm_gate(q, k, v, g, gate[:, :-1], w)
+    with pytest.raises(AssertionError, match="dtype of q"):
+        forgetting_attention_norm_gate(q, k, v, g, gate.half() if q.dtype == torch.bfloat16 else gate.bfloat16(), w)
+    with pytest.raises(ValueError, match="Unsupported activation"):
+        forgetting_attention_norm_gate(q, k, v, g, gate, w, activation="relu")
+    with pytest.raises(AssertionError, match="Only torch.float16 or torch.bfloat16"):
+        forgetting_attention_norm_gate(q.float(), k, v, g, gate, w)
+    lib = _lib.load()
+    args, epi = _lib.FwdArgs(), _lib.FwdEpilogue()
+    assert lib.fox_attn_fwd_norm_gate(None, C.byref(epi), None) != 0
+    assert lib.fox_attn_fwd_norm_gate(C.byref(args), None, None) != 0
+    epi.activation = 7
+    assert lib.fox_attn_fwd_norm_gate(C.byref(args), C.byref(epi), None) != 0
+    assert b"activation" in lib.fox_last_error()
+    epi.activation = _lib.ACT_NONE
+    assert lib.fox_attn_fwd_norm_gate(C.byref(args), C.byref(epi), None) != 0
+    assert b"y is NULL" in lib.fox_last_error()
+
+
 def test_product_code_never_touches_the_oracle():
     pkg = ROOT / "forgetting-transformer_amd"
     for path in list(pkg.rglob("*.py")) + list(pkg.rglob("*.hip")) + list(pkg.rglob("*.hpp")):
