@@ -359,7 +359,8 @@ __device__ __forceinline__ void store_rows_norm_gate(char* stage, const f32x16 (
         float y1 = Tr::hi(xv[e]) * rs * (e < 2 ? w0[2 * e + 1] : w1[2 * e - 3]);
         if (act != kActNone) {
           const float g0 = Tr::lo(gv[e]), g1 = Tr::hi(gv[e]);
-          const float s0 = sigmoidf(g0), s1 = sigmoidf(g1);
+          // (hardware reciprocal, one unit in the last place: this loop sits at the tail of a workgroup's critical path)
+          const float s0 = __builtin_amdgcn_rcpf(1.0f + __expf(-g0)), s1 = __builtin_amdgcn_rcpf(1.0f + __expf(-g1));
           y0 *= act == kActSwish ? g0 * s0 : s0;
           y1 *= act == kActSwish ? g1 * s1 : s1;
         }
