@@ -28,11 +28,16 @@ def pytest_configure(config):
 #             rounding noise of a 16-bit result is about uniform over rows, half an ulp of the largest element
 #             alone is 2e-3 of the scale), so a wrong small row cannot hide behind a large one elsewhere.
 # Every measured ratio is kept and the worst per output is printed at the end of the run, so the margin
-# against the bar is on record.
+# against the bar is on record; TRIPWIRE turns a margin that shrinks into a failure.
 # --------------------------------------------------------------------------------------
 REL_TOL = 2e-2
 ROW_RTOL = 2e-2
 ROW_ATOL = 6e-3
+# Regression tripwire under the bar: about 1.5 x the worst ratio any case of the suite has measured for that output
+# (the kernels are deterministic, so the ratios repeat run to run).  A check at the standard bar that lands between
+# its tripwire and the bar fails with a message of its own: either the kernels' error grew, or the new case is
+# noisier than every case before it -- look before raising the figure.
+TRIPWIRE = {"out": 8e-3, "dq": 1.4e-2, "dk": 1.1e-2, "dv": 7e-3, "dlog_fgate": 8.5e-3, "dc_steps": 8.5e-3}
 _MARGINS = {}
 
 
@@ -77,6 +82,9 @@ def assert_parity(name, x, ref, tol=REL_TOL, rows=True, context=None, floor=0.0)
     std = tol == REL_TOL and floor == 0.0
     e = rel_err(x, ref, name if std else None, floor)
     assert e <= tol, f"{name}: max-abs error / scale = {e:.3e} > {tol:.3e} {context or ''}"
+    if std and name in TRIPWIRE:
+        assert e <= TRIPWIRE[name], (f"{name}: max-abs error / scale = {e:.3e} is within the bar {tol:.1e} but above the "
+                                     f"regression tripwire {TRIPWIRE[name]:.1e} {context or ''}")
     if rows:
         r = row_err(x, ref, name if std else None, scale=max(1.0, tol / REL_TOL), floor=floor)
         assert r <= 1.0, f"{name}: worst row error = {r:.3f} of its bound {context or ''}"

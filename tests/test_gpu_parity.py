@@ -5,7 +5,9 @@ Tolerance (bf16): max |x - ref| <= 2e-2 * max|ref| for out, dq, dk, dv, dlog_fga
 configurations are judged by ("max-abs error 2e-2 relative to output scale"; the scale is the reference's own
 maximum, without a floor, unless the reference is exactly zero everywhere -- a single valid key per row gives
 dS = 0 exactly), and row by row for out, dq, dk, dv: |x - ref| <= 2e-2 * max|ref row| + 6e-3 * max|ref|, so
-a wrong row of small magnitude cannot hide behind a large one.  The measured ratios are printed at the end of the run.  The reference's own grid
+a wrong row of small magnitude cannot hide behind a large one.  dlog_fgate is a reverse running sum whose early
+entries dominate its scale, so its steps dc[n] = dlog_fgate[n] - dlog_fgate[n+1] are held to the same tensor-wide
+bar as well ("dc_steps").  The measured ratios are printed at the end of the run.  The reference's own grid
 (fp16) uses its own bound, atol = 1e-2 (ops/forgetting_attention.py:1416-1425).
 """
 import ctypes as C
@@ -47,7 +49,19 @@ def run_case(fa, B, H, M, N, D, *, dtype=torch.bfloat16, head_first=True, thr=No
             assert err <= atol, f"{name}: abs err {err:.3e} > {atol}"
         else:
             assert_parity(name, x, r, tol=tol, rows=name != "dlog_fgate")
+    if atol is None and tol == REL_TOL:
+        assert_parity("dc_steps", gate_grad_steps(g.grad, head_first), gate_grad_steps(ref[4], head_first), rows=False)
     return got, ref, ss
+
+
+def gate_grad_steps(dg, head_first):
+    """dc[n] = dg[n] - dg[n+1] (dc[N-1] = dg[N-1]): the gradient with respect to the cumulative sum, position by
+    position.  dlog_fgate is its reverse running sum, whose large early entries set the scale of the tensor-wide bound;
+    the steps put every position on the scale of its own row and column sums of dS."""
+    dg = dg.float()
+    axis = -1 if head_first else 1
+    last = dg.narrow(axis, dg.shape[axis] - 1, 1)
+    return torch.cat([-dg.diff(dim=axis), last], dim=axis)
 
 
 # --------------------------------------------------------------------------------------
@@ -525,6 +539,8 @@ def _full_size_check(fa, B, H, T, D, mean, std, thr, pairs, seq_start=None):
         for name, x, r in zip(("out", "dq", "dk", "dv"), got, ref):
             assert_parity(name, sl(x), r, context=(b, h))
         assert_parity("dlog_fgate", gates.grad[b:b + 1, :, h:h + 1], ref[4], rows=False, context=(b, h))
+        assert_parity("dc_steps", gate_grad_steps(gates.grad[b:b + 1, :, h:h + 1], False), gate_grad_steps(ref[4], False),
+                      rows=False, context=(b, h))
     return out.detach()
 
 
