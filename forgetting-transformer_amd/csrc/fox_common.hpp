@@ -50,6 +50,11 @@ struct Bf16 {
   }
   static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
   static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+  // acc + lo(w) + hi(w) in one instruction (v_dot2c_f32_bf16 against a pair of ones)
+  static __device__ __forceinline__ float add_pair(uint32_t w, float acc) {
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, acc, false);
+  }
 };
 
 struct Fp16 {
@@ -62,6 +67,10 @@ struct Fp16 {
   }
   static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
   static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
+  static __device__ __forceinline__ float add_pair(uint32_t w, float acc) {
+    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, acc, false);
+  }
 };
 
 // Pack eight consecutive accumulator values into one 16-byte MFMA operand.

@@ -84,27 +84,26 @@ __device__ __forceinline__ void fwd_tile(const char* k_tile, const char* v_tile,
 #pragma unroll
       for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
   }
-  float rsum = 0.f;
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float p = __builtin_amdgcn_exp2f(s[nb][r] - m_i);
-      s[nb][r] = p;
-      rsum += p;
-    }
-  l_i += rsum;  // per-lane partial sum; the two halves are added in the epilogue
+    for (int r = 0; r < 16; ++r) s[nb][r] = __builtin_amdgcn_exp2f(s[nb][r] - m_i);
 
-  // O^T += V^T P^T
+  // O^T += V^T P^T.  The row sum is taken over the probabilities as rounded for the MFMA (the weights that
+  // multiply V then add up to exactly l), two at a time: per-lane partial sum, the two halves are added in the epilogue.
+  float rsum = 0.f;
 #pragma unroll
   for (int sl = 0; sl < BN / 16; ++sl) {
     const u32x4 pb = pack8<Tr>(s[sl >> 1], 8 * (sl & 1));
+#pragma unroll
+    for (int e = 0; e < 4; ++e) rsum = Tr::add_pair(pb[e], rsum);
     u32x4 va[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) va[db] = lds_col_operand<D>(v_tile, 16 * sl, db, lane);
 #pragma unroll
     for (int db = 0; db < DB; ++db) oacc[db] = Tr::mfma32(va[db], pb, oacc[db]);
   }
+  l_i += rsum;
 }
 
 // Interior tile (no key of the tile is right of any query row of the workgroup): branch-free and
@@ -185,18 +184,16 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
     if (c < NSL) {
       const int nb = c >> 1, r0 = 8 * (c & 1);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float p = __builtin_amdgcn_exp2f(fmaf(s_cur[nb][r0 + e], qk_scale, neg_m));
-        s_cur[nb][r0 + e] = p;
-        rsum += p;
-      }
+      for (int e = 0; e < 8; ++e) s_cur[nb][r0 + e] = __builtin_amdgcn_exp2f(fmaf(s_cur[nb][r0 + e], qk_scale, neg_m));
       pb[c] = pack8<Tr>(s_cur[nb], r0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) rsum = Tr::add_pair(pb[c][e], rsum);  // row sum of the rounded probabilities
     }
     if (c >= 1 && c < NSL) {
 #pragma unroll
-      for (int k = 0; k < DB; ++k) {  // a slice has 20 vector and 8 exp instructions: dealt out over its DB MFMAs
+      for (int k = 0; k < DB; ++k) {  // a slice has 16 vector and 8 exp instructions: dealt out over its DB MFMAs
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 20 / DB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 16 / DB, 0);
         __builtin_amdgcn_sched_group_barrier(0x400, 8 / DB, 0);
       }
     }
@@ -235,8 +232,13 @@ struct TileDma {
 
 // EPI: the variant whose epilogue also applies the layer's output norm and gate (a.epi); a variant of its own so
 // that the plain kernel's register allocation is not touched by it.
+// Waves per SIMD the forward is compiled for: the register budget that goes with it (512 / waves) holds the
+// kernel to the occupancy its head dim allows.
+template <int D>
+constexpr int kFwdWaves = D <= 64 ? 3 : 2;
+
 template <typename Tr, int D, bool SPLIT, bool EPI = false>
-__global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdK a) {
+__global__ __launch_bounds__(256, kFwdWaves<D>) void fwd_kernel(const FwdK a) {
   static_assert(!(SPLIT && EPI), "partial results of a key split are not normalised");
   constexpr int BM = kFwdBM, BN = kFwdBN;
   constexpr int KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;

@@ -37,7 +37,7 @@ ROW_ATOL = 6e-3
 # (the kernels are deterministic, so the ratios repeat run to run).  A check at the standard bar that lands between
 # its tripwire and the bar fails with a message of its own: either the kernels' error grew, or the new case is
 # noisier than every case before it -- look before raising the figure.
-TRIPWIRE = {"out": 8e-3, "dq": 1.4e-2, "dk": 1.1e-2, "dv": 7e-3, "dlog_fgate": 8.5e-3, "dc_steps": 8.5e-3}
+TRIPWIRE = {"out": 6e-3, "dq": 1.4e-2, "dk": 1.1e-2, "dv": 7e-3, "dlog_fgate": 8.5e-3, "dc_steps": 8.5e-3}
 _MARGINS = {}
 
 
