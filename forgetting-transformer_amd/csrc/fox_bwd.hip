@@ -333,7 +333,8 @@ __global__ __launch_bounds__(256, (D <= 64 || DSPLIT) ? 2 : 1) void dkdv_kernel(
   if (n0 + BN <= seq) m_hi = m_lo;  // every key of the tile is left padding
   const int n_steps = m_hi > m_lo ? (m_hi - m_lo + BMQ - 1) / BMQ : 0;
 
-  // Phase 1: the steps that touch the tile's diagonal (at most BN/BMQ + 1 of them) run one at a
+  // The long-loop kernel (head dim 128, one workgroup per CU).  Phase 1: the steps that touch the tile's
+  // diagonal (at most BN/BMQ + 1 of them) run one at a
   // time through buffer 1 with the masking code; the first interior tile is requested into
   // buffer 0 before the last of them is computed.  Phase 2: interior steps, double-buffered,
   // from the end of the sequence down: the workgroups of one (batch, head) that run together on
@@ -342,6 +343,30 @@ __global__ __launch_bounds__(256, (D <= 64 || DSPLIT) ? 2 : 1) void dkdv_kernel(
   int n_diag = 0;
   while (n_diag < n_steps && p_seq + m_lo + n_diag * BMQ < n0 + BN - 1) ++n_diag;
   const int n_int = n_steps - n_diag, m_top = m_lo + (n_steps - 1) * BMQ;
+  if constexpr (D <= 64 || DSPLIT) {
+    // Small head dims (and the split variant) leave room for two workgroups per CU: the second wave on each SIMD
+    // fills the matrix pipe while the first does its vector work, so every step takes the plain code path.  The
+    // steps, diagonal ones first (upwards from m_lo), then the interior ones (downwards from m_top), alternate
+    // between the two buffer sets, starting with set 1 (which the early request above has filled): the next step's
+    // tiles are requested before the current one is computed.
+    auto step_rows = [&](int idx) { return idx < n_diag ? m_lo + idx * BMQ : m_top - (idx - n_diag) * BMQ; };
+    if (n_steps > 0) {
+      if (!early) issue(step_rows(0), q_tile1, do_tile1);
+      if (row_lane) { rc_s1[row_slot] = rc_term(); dl_s1[row_slot] = dl_term(); }
+    }
+    for (int idx = 0; idx < n_steps; ++idx) {
+      const bool odd = idx & 1;
+      wait_vmem_all();
+      __syncthreads();
+      if (idx + 1 < n_steps) issue(step_rows(idx + 1), odd ? q_tile1 : q_tile0, odd ? do_tile1 : do_tile0);
+      dkdv_step<Tr, D, BMQ, NDB>(odd ? q_tile0 : q_tile1, odd ? do_tile0 : do_tile1, odd ? rc_s0 : rc_s1, odd ? dl_s0 : dl_s1, kreg,
+                                 vreg, dkacc, dvacc, csum, p_seq + step_rows(idx), n, n_w0, qk_scale, colc, lane, dh * NDB);
+      if (idx + 1 < n_steps && row_lane) {
+        (odd ? rc_s1 : rc_s0)[row_slot] = rc_term();
+        (odd ? dl_s1 : dl_s0)[row_slot] = dl_term();
+      }
+    }
+  } else {
   for (int t = 0; t < n_diag; ++t) {
     const int ms = m_lo + t * BMQ;
     if (!(early && t == 0)) {
@@ -359,23 +384,6 @@ __global__ __launch_bounds__(256, (D <= 64 || DSPLIT) ? 2 : 1) void dkdv_kernel(
     if (n_diag == 0) issue(m_top, q_tile0, do_tile0);
     if (row_lane) { rc_s0[row_slot] = rc_term(); dl_s0[row_slot] = dl_term(); }
   }
-  if constexpr (D <= 64 || DSPLIT) {
-    // Small head dims (and the split variant) leave room for two workgroups per CU: the second wave on each SIMD
-    // fills the matrix pipe while the first does its vector work, so the plain step is used for interior tiles too.
-    for (int t = 0; t < n_int; ++t) {
-      const bool odd = t & 1;
-      wait_vmem_all();
-      __syncthreads();
-      if (t + 1 < n_int) issue(m_top - (t + 1) * BMQ, odd ? q_tile0 : q_tile1, odd ? do_tile0 : do_tile1);
-      const int ms = m_top - t * BMQ;
-      dkdv_step<Tr, D, BMQ, NDB>(odd ? q_tile1 : q_tile0, odd ? do_tile1 : do_tile0, odd ? rc_s1 : rc_s0, odd ? dl_s1 : dl_s0, kreg,
-                                 vreg, dkacc, dvacc, csum, p_seq + ms, n, n_w0, qk_scale, colc, lane, dh * NDB);
-      if (t + 1 < n_int && row_lane) {
-        (odd ? rc_s0 : rc_s1)[row_slot] = rc_term();
-        (odd ? dl_s0 : dl_s1)[row_slot] = dl_term();
-      }
-    }
-  } else {
   constexpr int PER = DirectTileLoader<D, BMQ>::PER;
   for (int t = 0; t < n_int; t += 2) {
     wait_vmem_all();
@@ -516,9 +524,18 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
   const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
   const int n0_first = hi > 0 ? ((hi - 1) / BN) * BN : 0;
   const bool early = hi > (min(seq, hi) / BN) * BN;
+  // The tile before it as well, when neither the pruning bound (it never cuts right of the first row's own
+  // position) nor seq_start can exclude it: under pruning a workgroup visits two or three tiles, and every round
+  // trip taken out of that chain counts.
+  const int n0_second = n0_first - BN;
+  const bool early2 = early && n0_second >= (a0 / BN) * BN && n0_second >= (min(seq, hi) / BN) * BN;
   if (early) {
     kld.issue(kp, a.k.st, n0_first, N, k_tile0);
     vld.issue(vp, a.v.st, n0_first, N, v_tile0);
+  }
+  if (early2) {
+    kld.issue(kp, a.k.st, n0_second, N, k_tile1);
+    vld.issue(vp, a.v.st, n0_second, N, v_tile1);
   }
   u32x4 qreg[KK], doreg[KK];
   load_row_operand_regs<D>(qreg, qp, a.q.st, m, M, g);
@@ -571,6 +588,13 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     vld.issue(vp, a.v.st, n0, N, vt);
   };
   if (early) issue_cn(n0_first);
+  float cn_raw2 = 0.f;   // key terms of the second early tile: handed to cn_raw once the first tile's are in LDS
+  bool cn_ok2 = false;
+  if (early2 && tid < BN) {
+    const int nn = n0_second + tid;
+    cn_ok2 = (nn < N) & (nn >= seq);
+    cn_raw2 = c_row[min(nn, N - 1)];
+  }
 
   int lo = min(seq, hi);
   if (a.thr) {
@@ -586,21 +610,25 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     dq_tile<Tr, D>(kt, vt, cn, qreg, doreg, dqacc, rsum, n0, a_m, a_w0, qk_scale, rowc, delta, lane);
   };
 
+  auto tile_n0 = [&](int t) { return lo + t * BN; };   // start of the tile at loop position t
   if (n_tiles > 0) {
-    if (!early) issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
+    if (!early) issue(tile_n0(n_tiles - 1), k_tile0, v_tile0);
     if (tid < BN) cn_s0[tid] = cn_term();
+    if (early2) { cn_raw = cn_raw2; cn_ok = cn_ok2; }
   }
+  bool requested = early2;  // buffers 1 already hold (or await) the next tile
   for (int t = n_tiles - 1; t >= 0; t -= 2) {
     wait_vmem_all();
     __syncthreads();
-    if (t >= 1) issue(lo + (t - 1) * BN, k_tile1, v_tile1);
-    compute(lo + t * BN, k_tile0, v_tile0, cn_s0);
+    if (t >= 1 && !requested) issue(tile_n0(t - 1), k_tile1, v_tile1);
+    requested = false;
+    compute(tile_n0(t), k_tile0, v_tile0, cn_s0);
     if (t < 1) break;
     if (tid < BN) cn_s1[tid] = cn_term();
     wait_vmem_all();
     __syncthreads();
-    if (t >= 2) issue(lo + (t - 2) * BN, k_tile0, v_tile0);
-    compute(lo + (t - 1) * BN, k_tile1, v_tile1, cn_s1);
+    if (t >= 2) issue(tile_n0(t - 2), k_tile0, v_tile0);
+    compute(tile_n0(t - 1), k_tile1, v_tile1, cn_s1);
     if (t >= 2 && tid < BN) cn_s0[tid] = cn_term();
   }
 

@@ -33,6 +33,7 @@
 namespace fox {
 
 constexpr float kLazyMaxLog2 = 8.0f;
+constexpr int kMinPipelinedTiles = 4;   // interior tiles below which the software-pipelined path is not entered
 
 template <typename Tr, int D>
 __device__ __forceinline__ void fwd_tile(const char* k_tile, const char* v_tile, const float* cn_s, const u32x4 (&qreg)[D / 16],
@@ -286,9 +287,19 @@ __global__ __launch_bounds__(256, kFwdWaves<D>) void fwd_kernel(const FwdK a) {
   const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
   const int n0_first = hi > 0 ? ((hi - 1) / BN) * BN : 0;
   const bool early = !SPLIT && hi > (min(seq, hi) / BN) * BN && (n0_first + BN - 1 > a0 || !(qk_scale > 0.f));
+  // The tile before it is requested as well when nothing can exclude it: it still reaches the workgroup's first row
+  // (the pruning bound never cuts there) and lies right of seq_start.  Under pruning a workgroup visits two or
+  // three tiles, and every round trip taken out of that chain counts.
+  const int n0_second = n0_first - BN;
+  const bool early2 = early && n0_second >= (a0 / BN) * BN && n0_second >= (min(seq, hi) / BN) * BN &&
+                      (n0_second + BN - 1 > a0 || !(qk_scale > 0.f));
   if (early) {
     kld.issue(kp, a.k.st, n0_first, N, k_tile0);
     vld.issue(vp, a.v.st, n0_first, N, v_tile0);
+  }
+  if (early2) {
+    kld.issue(kp, a.k.st, n0_second, N, k_tile1);
+    vld.issue(vp, a.v.st, n0_second, N, v_tile1);
   }
   u32x4 qreg[KK];
   load_row_operand_regs<D>(qreg, qp, a.q.st, m, M, g);
@@ -314,6 +325,13 @@ __global__ __launch_bounds__(256, kFwdWaves<D>) void fwd_kernel(const FwdK a) {
     vld.issue(vp, a.v.st, n0, N, vt);
   };
   if (early) issue_cn(n0_first);
+  float cn_raw2 = 0.f;   // key terms of the second early tile: handed to cn_raw once the first tile's are in LDS
+  bool cn_ok2 = false;
+  if (early2 && tid < BN) {
+    const int n = n0_second + tid;
+    cn_ok2 = (n < N) & (n >= seq);
+    cn_raw2 = c_row[min(n, N - 1)];
+  }
   const float cm2 = (m < M) ? (c_m - c_ref) * kLog2e : 0.f;
 
   f32x16 oacc[DB];
@@ -353,24 +371,31 @@ __global__ __launch_bounds__(256, kFwdWaves<D>) void fwd_kernel(const FwdK a) {
   int n_diag = 0;
   while (n_diag < n_tiles && lo + (n_tiles - 1 - n_diag) * BN + BN - 1 > a0) ++n_diag;
   if (!(qk_scale > 0.f)) n_diag = n_tiles;
+  // The pipelined path starts with two round trips of its own (K of its first tile, then V): worth it for a long
+  // walk only.  With a few interior tiles (the usual case under pruning) they go through phase 1 as well.
+  if (n_tiles - n_diag < kMinPipelinedTiles) n_diag = n_tiles;
   const int t_stop = n_tiles - n_diag;
+  auto tile_n0 = [&](int t) { return lo + t * BN; };   // start of the tile at loop position t
   if (n_diag > 0) {
-    if (!early) issue(lo + (n_tiles - 1) * BN, k_tile0, v_tile0);
+    if (!early) issue(tile_n0(n_tiles - 1), k_tile0, v_tile0);
     if (tid < BN) cn_s0[tid] = cn_term();
+    if (early2) { cn_raw = cn_raw2; cn_ok = cn_ok2; }
   }
+  bool requested = early2;  // buffers 1 already hold (or await) the next tile
   for (int t = n_tiles - 1; t >= t_stop; t -= 2) {
     // even step: consume buffers 0, fill buffers 1
     wait_vmem_all();
     __syncthreads();
-    if (t - 1 >= t_stop) issue(lo + (t - 1) * BN, k_tile1, v_tile1);
-    compute(lo + t * BN, k_tile0, v_tile0, cn_s0);
+    if (t - 1 >= t_stop && !requested) issue(tile_n0(t - 1), k_tile1, v_tile1);
+    requested = false;
+    compute(tile_n0(t), k_tile0, v_tile0, cn_s0);
     if (t - 1 < t_stop) break;
     if (tid < BN) cn_s1[tid] = cn_term();
     // odd step: consume buffers 1, fill buffers 0
     wait_vmem_all();
     __syncthreads();
-    if (t - 2 >= t_stop) issue(lo + (t - 2) * BN, k_tile0, v_tile0);
-    compute(lo + (t - 1) * BN, k_tile1, v_tile1, cn_s1);
+    if (t - 2 >= t_stop) issue(tile_n0(t - 2), k_tile0, v_tile0);
+    compute(tile_n0(t - 1), k_tile1, v_tile1, cn_s1);
     if (t - 2 >= t_stop && tid < BN) cn_s0[tid] = cn_term();
   }
 
