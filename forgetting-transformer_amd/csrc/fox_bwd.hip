@@ -537,37 +537,13 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     kld.issue(kp, a.k.st, n0_second, N, k_tile1);
     vld.issue(vp, a.v.st, n0_second, N, v_tile1);
   }
-  u32x4 qreg[KK], doreg[KK];
+  u32x4 qreg[KK], doreg[KK], oreg[KK];
   load_row_operand_regs<D>(qreg, qp, a.q.st, m, M, g);
   load_row_operand_regs<D>(doreg, dop, a.d_o.st, m, M, g);
+  load_row_operand_regs<D>(oreg, op, a.o.st, m, M, g);
   const float c_ref = c_row[a0];
-  // rows past M and empty rows (lse = -inf) get rowc = -inf through the subtraction: no load behind a branch
   const int mc = min(m, M - 1);
   const float l = a.lse[(int64_t)bh * M + mc], c_m = c_row[min(p_seq + mc, N - 1)];
-  const float l_eff = ((m < M) & (l > -INFINITY)) ? l : INFINITY;
-  const float rowc = (c_m - c_ref - l_eff) * kLog2e;
-  // delta_i = sum_d o_id * do_id (_bwd_preprocess of the reference, :902-943) for this lane's row: each half of
-  // the wave holds half of the row's elements.  Rows past M were loaded as zeros.  Stored for the dK/dV kernel.
-  float delta;
-  {
-    u32x4 oreg[KK];
-    load_row_operand_regs<D>(oreg, op, a.o.st, m, M, g);
-    float part = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk)
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        part += Tr::lo(oreg[kk][e]) * Tr::lo(doreg[kk][e]) + Tr::hi(oreg[kk][e]) * Tr::hi(doreg[kk][e]);
-    delta = half_sum(part);
-    if (m < M && g == 0) a.delta[(int64_t)bh * M + m] = delta;
-  }
-
-  f32x16 dqacc[DB];
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
-  float rsum = 0.f;
 
   // Key terms of a tile: the load is requested here, the arithmetic on it is done where the value goes to
   // LDS (a tile later), so that nothing waits for the load in between.  Masked keys get -inf through the
@@ -596,6 +572,8 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     cn_raw2 = c_row[min(nn, N - 1)];
   }
 
+  // The pruning bound: its loads are the last to join the ones above, and the search's first wait is the wait for
+  // all of them.  Nothing before this point waits for a load: one round trip covers the whole prologue.
   int lo = min(seq, hi);
   if (a.thr) {
     const int t = acp_first_kept_block(c_row, c_ref, a.thr[bh], N, BN, a0 / BN, lane);
@@ -603,6 +581,30 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
   }
   lo = (lo / BN) * BN;
   const int n_tiles = (hi - lo + BN - 1) / BN;
+
+  // rows past M and empty rows (lse = -inf) get rowc = -inf through the subtraction: no load behind a branch
+  const float l_eff = ((m < M) & (l > -INFINITY)) ? l : INFINITY;
+  const float rowc = (c_m - c_ref - l_eff) * kLog2e;
+  // delta_i = sum_d o_id * do_id (_bwd_preprocess of the reference, :902-943) for this lane's row: each half of
+  // the wave holds half of the row's elements.  Rows past M were loaded as zeros.  Stored for the dK/dV kernel.
+  float delta;
+  {
+    float part = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        part += Tr::lo(oreg[kk][e]) * Tr::lo(doreg[kk][e]) + Tr::hi(oreg[kk][e]) * Tr::hi(doreg[kk][e]);
+    delta = half_sum(part);
+    if (m < M && g == 0) a.delta[(int64_t)bh * M + m] = delta;
+  }
+
+  f32x16 dqacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
+  float rsum = 0.f;
 
   const bool wave_has_rows = m0 + 32 * wave < M;  // a wave without query rows only moves tiles
   auto compute = [&](int n0, const char* kt, const char* vt, const float* cn) {
