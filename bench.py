@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Forgetting Attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode|c3d64|c3d32|c3d16|shift|norm_gate|ref_sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode|c3d64|c3d32|c3d16|shift|norm_gate|ref_sweep|acp_sweep]
                     [--no-extras] [--no-cpu-baseline]
 
 A step is one forward + backward pass of ``forgetting_attention`` over one batch
@@ -501,6 +501,45 @@ def ref_sweep_report(ns):
         "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS, "sweep": rows}))
 
 
+def acp_sweep_report(ns):
+    """Speed-up of the pruned step against the unpruned one on the same inputs, as a function of how much pruning
+    keeps: config 4's shape with constant gates -10/W, so that with adaptive_threshold = -10 every query row keeps a
+    band of W keys (W * T - W^2 / 2 of the T^2 / 2 causal pairs).  One JSON line."""
+    from forgetting_transformer import forgetting_attention
+
+    w = dict(WORKLOADS["c4"])
+    q, k, v, g, do, _ = synth(w, "cuda", seed=1)
+    q, k, v = (x.requires_grad_() for x in (q, k, v))
+    T = w["N"]
+    steps, warmup = max(3, ns.steps // 2), 2
+
+    def step(gates, thr):
+        out = forgetting_attention(q, k, v, gates, adaptive_threshold=thr)
+        out.backward(do)
+        q.grad = k.grad = v.grad = gates.grad = None
+
+    rows = []
+    for W in (128, 256, 512, 1024, 2048, 4096, 8192):
+        gates = torch.full_like(g, -10.0 / W).requires_grad_()
+        t_full = time_steps(lambda: step(gates, None), steps, warmup)
+        t_acp = time_steps(lambda: step(gates, -10.0), steps, warmup)
+        st = stage_times(w, (q.detach(), k.detach(), v.detach(), gates.detach(), do, None), steps, threshold=-10.0)
+        kept = (W * T - W * W / 2.0) / (T * T / 2.0)
+        rows.append({"band_keys": W, "kept_fraction": kept, "ms_unpruned": t_full * 1e3, "ms_pruned": t_acp * 1e3,
+                     "speedup": t_full / t_acp, "proportional_speedup": 1.0 / kept,
+                     "fraction_of_proportional": (t_full / t_acp) * kept,
+                     "kernels_ms": {name: st[name] * 1e3 for name in ("fwd", "bwd_dq", "bwd_dkdv")}})
+    line = {
+        "metric": "ACP speed-up vs no-prune on the same inputs, by kept fraction", "value": rows[0]["speedup"], "unit": "x",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": rows[0]["ms_pruned"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"acp_sweep: B{w['B']} T{T} H{w['H']} D{w['D']} bf16 fwd+bwd, constant gates -10/W, "
+                               "adaptive_threshold -10, W = kept band in keys"},
+        "sweep": rows,
+    }
+    print(json.dumps(line))
+
+
 def shift_report(ns):
     """Token shift (the key/value pre-processing of the FoX layer) at the training-layer shape:
     forward + backward, HBM-bound; one JSON line of its own."""
@@ -638,7 +677,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift", "norm_gate", "ref_sweep"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift", "norm_gate", "ref_sweep", "acp_sweep"])
     ap.add_argument("--threshold", default=None,
                     help="adaptive_threshold of the main workload: a float or 'auto' (default: no pruning); with it the "
                          "roofline entry prices the dK/dV pass against HBM, the bound of a heavily pruned step")
@@ -667,6 +706,8 @@ def main():
         return shift_report(ns)
     if ns.workload == "norm_gate":
         return norm_gate_report(ns)
+    if ns.workload == "acp_sweep":
+        return acp_sweep_report(ns)
     if ns.workload == "ref_sweep":
         return ref_sweep_report(ns)
 
