@@ -510,6 +510,36 @@ def test_long_sequences_at_small_head_dims(fa, D, M, N, seq, thr):
 
 
 # --------------------------------------------------------------------------------------
+# a sequence longer than any benchmark configuration, through properties that need no full-size oracle
+# --------------------------------------------------------------------------------------
+def test_sequence_of_65536_tokens(fa):
+    """T = 65536 (512 query tiles, 1024 key tiles per head).  Causality: the first 8192 rows of the output must equal,
+    bit for bit, the output on the first 8192 tokens alone (same tiles in the same order).  Under strong decay
+    (gate logits N(-1, 1): a key 200 positions back weighs less than e^-100) the last rows and keys only see the last
+    few thousand tokens, so the oracle on that window pins out, dq, dk, dv and the steps of dlog_fgate there (a constant
+    shift of the cumulative sums cancels in every c_i - c_j)."""
+    B, H, T, D, W = 1, 8, 65536, 64, 4096    # 8 heads: enough query tiles that neither run splits its key loops
+    q, k, v, g, do, _ = make_inputs(B, H, T, T, D, dtype=torch.bfloat16, device="cuda", head_first=False, seed=77,
+                                    gate_mean=-1.0, gate_std=1.0)
+    q, k, v, g = (x.requires_grad_() for x in (q, k, v, g))
+    out = fa(q, k, v, g)
+    out.backward(do)
+    for x in (out, q.grad, k.grad, v.grad, g.grad):
+        assert torch.isfinite(x).all()
+    assert (g.grad[:, 0] == 0).all()
+    with torch.no_grad():
+        head = fa(q[:, :8192], k[:, :8192], v[:, :8192], g[:, :8192])
+    assert torch.equal(out[:, :8192], head)
+    lo = T - W
+    ref = O.forgetting_attention_ref_grads(q.detach()[:, lo:], k.detach()[:, lo:], v.detach()[:, lo:], g.detach()[:, lo:], do[:, lo:],
+                                           bh_chunk=2)
+    half = W // 2   # rows / keys of the window whose whole reach lies inside it
+    for name, x, r in zip(("out", "dq", "dk", "dv"), (out, q.grad, k.grad, v.grad), ref):
+        assert_parity(name, x[:, lo + half:], r[:, half:], context="last rows of 65536")
+    assert_parity("dc_steps", gate_grad_steps(g.grad[:, lo + half:], False), gate_grad_steps(ref[4][:, half:], False), rows=False)
+
+
+# --------------------------------------------------------------------------------------
 # benchmark configurations 3-5 at full size
 # --------------------------------------------------------------------------------------
 # One (batch, head) pair per XCD: the workgroup -> (batch, head) map of the kernels puts pair bh on XCD bh mod 8,
