@@ -578,6 +578,33 @@ def test_config3_long_context(fa):
     _full_size_check(fa, 4, 16, 16384, 128, 3.0, 1.0, None, ALL_XCD_PAIRS)
 
 
+@pytest.mark.parametrize("thr", [None, -10.0])
+def test_config3_results_do_not_depend_on_where_a_head_sits(fa, thr):
+    """Every (batch, head) pair is an independent problem, and the kernels map pair bh to XCD bh mod 8 and to a
+    position in the launch order.  Rotating the batch by one and the heads by three moves every pair to another XCD
+    and another place in the grid; all five outputs of all 64 pairs must come out bit for bit the same (with the
+    oracle on one pair per XCD above, that extends to every pair what those eight pin).  Also under pruning, with
+    config 4's gates."""
+    B, H, T, D = 4, 16, 16384, 128
+    g_ = torch.Generator(device="cuda").manual_seed(5)
+    mean, std = (3.0, 1.0) if thr is None else (-1.0, 2.0)
+    q, k, v = (torch.randn(B, T, H, D, generator=g_, device="cuda").bfloat16() for _ in range(3))
+    gates = F.logsigmoid(torch.randn(B, T, H, generator=g_, device="cuda") * std + mean)
+    do = torch.randn(B, T, H, D, generator=g_, device="cuda").bfloat16()
+    rot = lambda x: torch.roll(x, shifts=(1, 3), dims=(0, 2)).contiguous()
+
+    def run(q, k, v, gates, do):
+        q, k, v, gates = (x.clone().requires_grad_() for x in (q, k, v, gates))
+        out = fa(q, k, v, gates, adaptive_threshold=thr)
+        out.backward(do)
+        return out.detach(), q.grad, k.grad, v.grad, gates.grad
+
+    a = run(q, k, v, gates, do)
+    b = run(rot(q), rot(k), rot(v), rot(gates), rot(do))
+    for name, x, y in zip(("out", "dq", "dk", "dv", "dlog_fgate"), a, b):
+        assert torch.equal(rot(x), y), name
+
+
 def test_config3_shape_with_left_padding(fa):
     """The long-context shape with left padding, forward and backward: padding inside the first tile, across many
     tiles, ending mid-tile just below the middle, and leaving only the last 300 positions."""
