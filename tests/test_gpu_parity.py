@@ -605,6 +605,24 @@ def test_config3_results_do_not_depend_on_where_a_head_sits(fa, thr):
         assert torch.equal(rot(x), y), name
 
 
+@pytest.mark.parametrize("M", [128, 1])
+def test_config5_results_do_not_depend_on_where_a_head_sits(fa, M):
+    """The same for the cache shapes (B16 H16 N32768 D128, head-first, left padding): the key-split forward, its
+    merge kernel and the single-query streaming kernel, every (batch, head) pair moved to another XCD."""
+    B, H, N, D = 16, 16, 32768, 128
+    g_ = torch.Generator(device="cuda").manual_seed(6)
+    q = torch.randn(B, H, M, D, generator=g_, device="cuda").bfloat16()
+    k, v = (torch.randn(B, H, N, D, generator=g_, device="cuda").bfloat16() for _ in range(2))
+    gates = F.logsigmoid(torch.randn(B, H, N, generator=g_, device="cuda") + 2.0)
+    ss = torch.randint(0, 8192, (B,), generator=g_, device="cuda")
+    rot = lambda x: torch.roll(x, shifts=(5, 3), dims=(0, 1)).contiguous()
+    with torch.no_grad():
+        a = fa(q, k, v, gates, head_first=True, seq_start=ss)
+        b = fa(rot(q), rot(k), rot(v), rot(gates), head_first=True, seq_start=torch.roll(ss, 5))
+    assert torch.isfinite(a).all()
+    assert torch.equal(rot(a), b)
+
+
 def test_config3_shape_with_left_padding(fa):
     """The long-context shape with left padding, forward and backward: padding inside the first tile, across many
     tiles, ending mid-tile just below the middle, and leaving only the last 300 positions."""
