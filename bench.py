@@ -381,9 +381,37 @@ def decode_report(steps, warmup):
     B, H, M, N, D = w["B"], w["H"], w["M"], w["N"], w["D"]
     pad = sets[0][5].float()
     alg = (2.0 * H * (N - pad) * D * 2).sum().item() + 2 * B * H * M * D * 2 + B * H * N * 4
-    return {"workload": "B16 M1 N32768 H16 D128 bf16 forward, head_first, seq_start~U[0,8192)",
-            "ms_per_step": t * 1e3, "kernel_ms": st["fwd"] * 1e3, "algorithmic_bytes": alg,
-            "kernel_hbm_gbps": alg / st["fwd"] * 1e-9, "kernel_frac_of_8TBps": alg / st["fwd"] * 1e-9 / PEAK_HBM_GBPS}
+    out = {"workload": "B16 M1 N32768 H16 D128 bf16 forward, head_first, seq_start~U[0,8192)",
+           "ms_per_step": t * 1e3, "kernel_ms": st["fwd"] * 1e3, "algorithmic_bytes": alg,
+           "kernel_hbm_gbps": alg / st["fwd"] * 1e-9, "kernel_frac_of_8TBps": alg / st["fwd"] * 1e-9 / PEAK_HBM_GBPS}
+
+    # The step as the layer runs it while generating: append the new token's key, value and gate to the cache, then
+    # attend.  The cache that grows in place copies the new token only; the reference's cache concatenates
+    # (fgate_cache.py:107-116), i.e. re-copies the layer's whole cache at every token.
+    from forgetting_transformer import FgateDynamicCache
+    q, k, v, log_fgate, _, ss = sets[0]
+    del sets
+    torch.cuda.empty_cache()
+    n0 = N - 64
+    k1, v1, g1 = k[:, :, n0:n0 + 1], v[:, :, n0:n0 + 1], log_fgate[:, :, n0:n0 + 1]
+    cache = FgateDynamicCache(max_length=N)
+    cache.update(k[:, :, :n0], v[:, :, :n0], log_fgate[:, :, :n0], 0)
+
+    def step_in_place():
+        cache.crop(n0)                       # the same position every time, so that all timed steps are alike
+        kk, vv, gg = cache.update(k1, v1, g1, 0)
+        forgetting_attention(q, kk, vv, gg, head_first=True, seq_start=ss)
+
+    state = [k[:, :, :n0].contiguous(), v[:, :, :n0].contiguous(), log_fgate[:, :, :n0].contiguous()]
+
+    def step_concatenating():
+        kk, vv, gg = torch.cat([state[0], k1], dim=2), torch.cat([state[1], v1], dim=2), torch.cat([state[2], g1], dim=2)
+        forgetting_attention(q, kk, vv, gg, head_first=True, seq_start=ss)
+
+    with torch.no_grad():
+        out["ms_per_step_with_cache_append"] = time_steps(step_in_place, steps, warmup) * 1e3
+        out["ms_per_step_with_concatenating_cache"] = time_steps(step_concatenating, steps, warmup) * 1e3
+    return out
 
 
 def head_dim_report(steps, warmup, name="c3d64"):
