@@ -278,8 +278,19 @@ __global__ __launch_bounds__(256, (D <= 64 || DSPLIT) ? 2 : 1) void dkdv_kernel(
     dold.issue(dop, a.d_o.st, m_lo, M, do_tile1);
   }
   u32x4 kreg[KK], vreg[KK];
-  load_row_operand_regs<D>(kreg, kp, a.k.st, n, N, g);
-  load_row_operand_regs<D>(vreg, vp, a.v.st, n, N, g);
+  // The split variant lives for two or three steps, so the way its K and V rows arrive counts: as register loads
+  // every instruction touches 32 rows for 32 bytes each; as tile loads they come in whole rows, through buffer set 0
+  // (free until the second step), and go from LDS to the registers like any row operand.
+  constexpr bool kStageKV = DSPLIT;
+  if constexpr (kStageKV) {
+    static_assert(BN == BMQ, "the key rows of a workgroup fill one step tile");
+    const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
+    kld.issue(kp, a.k.st, n0, N, q_tile0);
+    vld.issue(vp, a.v.st, n0, N, do_tile0);
+  } else {
+    load_row_operand_regs<D>(kreg, kp, a.k.st, n, N, g);
+    load_row_operand_regs<D>(vreg, vp, a.v.st, n, N, g);
+  }
   const float c_ref = c_row[n0];
   const float c_key = c_row[min(n, N - 1)];
   const float c_last = c_row[min(N - 1, n0 + BN - 1)];  // for the pruning bound below
@@ -332,6 +343,16 @@ __global__ __launch_bounds__(256, (D <= 64 || DSPLIT) ? 2 : 1) void dkdv_kernel(
   }
   if (n0 + BN <= seq) m_hi = m_lo;  // every key of the tile is left padding
   const int n_steps = m_hi > m_lo ? (m_hi - m_lo + BMQ - 1) / BMQ : 0;
+  if constexpr (kStageKV) {
+    wait_vmem_all();
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      kreg[kk] = lds_row_operand<D>(q_tile0, 32 * kb + i, 2 * kk + g);
+      vreg[kk] = lds_row_operand<D>(do_tile0, 32 * kb + i, 2 * kk + g);
+    }
+    __syncthreads();   // buffer set 0 is free for the second step's tiles
+  }
 
   // The long-loop kernel (head dim 128, one workgroup per CU).  Phase 1: the steps that touch the tile's
   // diagonal (at most BN/BMQ + 1 of them) run one at a
