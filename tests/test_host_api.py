@@ -25,6 +25,41 @@ def test_library_exports_every_declared_symbol():
     assert lib.fox_version() >= 100
 
 
+def test_public_header_is_plain_c(tmp_path):
+    """include/fox_attn.h must be usable from C and from C++ as it stands (the boundary is a C ABI): it compiles,
+    warning-free, as C99 and as C++11, and a C program that uses it links against the library and runs its host-only
+    calls (no device needed: version, tile table, an argument check that fails before any launch)."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no host C compiler")
+    src = tmp_path / "use_header.c"
+    src.write_text(f"""
+#include <stdio.h>
+#include <string.h>
+#include "{ROOT / 'include' / 'fox_attn.h'}"
+int main(void) {{
+  int32_t bm = 0, bn = 0, kn = 0, km = 0;
+  fox_fwd_args args;
+  memset(&args, 0, sizeof args);
+  if (fox_version() < 100) return 1;
+  if (fox_tile_config(128, &bm, &bn, &kn, &km) != FOX_OK || bm <= 0 || bn <= 0) return 2;
+  if (fox_tile_config(48, &bm, &bn, &kn, &km) == FOX_OK) return 3;
+  if (fox_attn_fwd(&args, NULL) == FOX_OK) return 4;      /* all-zero dims: rejected on the host */
+  if (strlen(fox_last_error()) == 0) return 5;
+  printf("%d %d\\n", bm, bn);
+  return 0;
+}}
+""")
+    for cmd in (["gcc", "-std=c99"], ["g++", "-std=c++11", "-x", "c++"]):
+        subprocess.run(cmd + ["-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", str(src)], check=True)
+    exe = tmp_path / "use_header"
+    lib_dir = _lib.LIB_PATH.parent
+    subprocess.run(["gcc", "-std=c99", str(src), "-o", str(exe), f"-L{lib_dir}", "-lfox_attn", f"-Wl,-rpath,{lib_dir}"], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert [int(x) for x in out] == list(_lib.tile_config(128)[:2])
+
+
 def test_kernels_do_not_spill():
     """The compiler's resource report, written next to the library by the build: the MFMA kernels must
     keep every register in the register file (a spill multiplies their run time) at the occupancy
