@@ -207,8 +207,8 @@ def stage_times(w, tensors, iters, threshold=None):
     dg = torch.empty_like(c)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     bwd = _lib.BwdArgs(dims, _view(q), _view(k), _view(v), _view(o), _view(dout), _view(dq), _view(dk), _view(dv),
-                       c.data_ptr(), lse.data_ptr(), ss, thr, 1.0 / math.sqrt(D), delta.data_ptr(), dc.data_ptr(),
-                       dg.data_ptr())
+                       c.data_ptr(), lse.data_ptr(), ss, thr, 1.0 / math.sqrt(D), delta[0].data_ptr(), delta[1].data_ptr(),
+                       dc.data_ptr(), dg.data_ptr())
     for name, fn in (("bwd_dq", lib.fox_attn_bwd_dq), ("bwd_dkdv", lib.fox_attn_bwd_dkdv)):
         out[name] = event_time(lambda fn=fn, name=name: _lib.check(fn(C.byref(bwd), stream), name), iters)
     out["cumsum_bwd"] = event_time(

@@ -342,6 +342,8 @@ __global__ __launch_bounds__(256, (D <= 64 || DSPLIT) ? 2 : 1) void dkdv_kernel(
     m_hi = min(M, u * BMQ);
   }
   if (n0 + BN <= seq) m_hi = m_lo;  // every key of the tile is left padding
+  if (a.kv_end_row && tid < BN / kKvUnit && n0 + tid * kKvUnit < N)  // the bound this workgroup works with, for callers that check it
+    a.kv_end_row[(int64_t)bh * ((N + kKvUnit - 1) / kKvUnit) + n0 / kKvUnit + tid] = m_hi;
   const int n_steps = m_hi > m_lo ? (m_hi - m_lo + BMQ - 1) / BMQ : 0;
   if constexpr (kStageKV) {
     wait_vmem_all();
@@ -601,6 +603,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdK a) {
     lo = max(lo, t * BN);
   }
   lo = (lo / BN) * BN;
+  if (a.q_first_block && tid == 0) a.q_first_block[(int64_t)bh * a.n_tiles + mt] = lo / BN;
   const int n_tiles = (hi - lo + BN - 1) / BN;
 
   // rows past M and empty rows (lse = -inf) get rowc = -inf through the subtraction: no load behind a branch

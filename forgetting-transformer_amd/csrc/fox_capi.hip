@@ -123,7 +123,7 @@ int make_bwd(const fox_bwd_args* args, fox::BwdK& k, bool need_grads) {
   k.o = to_view(args->o);
   k.d_o = to_view(args->d_o);
   k.delta = args->delta;
-  k.drow = args->delta + (int64_t)args->dims.B * args->dims.H * args->dims.M;
+  k.drow = args->drow;
   k.B = args->dims.B; k.H = args->dims.H; k.M = args->dims.M; k.N = args->dims.N;
   k.sm_scale = args->sm_scale;
   k.n_tiles = 0;
@@ -136,6 +136,8 @@ int make_bwd(const fox_bwd_args* args, fox::BwdK& k, bool need_grads) {
   FOX_TRY(check_extent(&args->k, args->dims.N, args->dims.D, "k"));
   FOX_TRY(check_extent(&args->v, args->dims.N, args->dims.D, "v"));
   if (!args->log_lambda || !args->lse || !args->dlog_lambda) return fail(FOX_E_ARG, "log_lambda, lse and dlog_lambda must not be NULL");
+  if (!args->drow) return fail(FOX_E_ARG, "drow is NULL");
+  if (args->drow == args->delta) return fail(FOX_E_ARG, "delta and drow must not alias");
   k.q = to_view(args->q);
   k.k = to_view(args->k);
   k.v = to_view(args->v);
@@ -144,6 +146,8 @@ int make_bwd(const fox_bwd_args* args, fox::BwdK& k, bool need_grads) {
   k.seq_start = args->seq_start;
   k.thr = args->threshold;
   k.dc = args->dlog_lambda;
+  k.q_first_block = args->q_first_block;
+  k.kv_end_row = args->kv_end_row;
   return FOX_OK;
 }
 
@@ -283,7 +287,7 @@ int fwd_impl(const fox_fwd_args* args, void* workspace, int64_t workspace_bytes,
 
 extern "C" {
 
-int fox_version(void) { return 100; }  // 0.1.0
+int fox_version(void) { return 200; }  // 0.2.0: fox_bwd_args and the scan entry points differ from 0.1.0
 
 const char* fox_last_error(void) { return g_err; }
 

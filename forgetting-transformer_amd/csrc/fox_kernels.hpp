@@ -51,7 +51,11 @@ struct BwdK {
   int n_tiles;
   int cls;         // kClassAll, or the class of key tiles this dK/dV launch handles (fox_common.hpp)
   int light_limit; // distance from the diagonal, in keys, that separates the two classes
+  int32_t* q_first_block;  // optional (B,H,ceil(M/kFwdBM)): first key block (of kFwdBN keys) each query tile of the dQ kernel visits
+  int32_t* kv_end_row;     // optional (B,H,ceil(N/kKvUnit)): per unit of kKvUnit keys, the query row at which the dK/dV kernel stops
 };
+
+constexpr int kKvUnit = 64;  // granularity of kv_end_row: the smallest key tile any dK/dV variant uses
 
 // Token shift: x, out, dout, dx are (B, T, H, D) 16-bit with shared element strides; the weights and
 // their gradients are (B, T, H) fp32 with shared element strides.

@@ -51,9 +51,12 @@ class BwdArgs(C.Structure):
         ("threshold", C.c_void_p),
         ("sm_scale", C.c_float),
         ("delta", C.c_void_p),
+        ("drow", C.c_void_p),
         ("dlog_lambda", C.c_void_p),
         ("dlog_fgate", C.c_void_p),
         ("dlog_fgate_stride_b", C.c_int64), ("dlog_fgate_stride_h", C.c_int64), ("dlog_fgate_stride_n", C.c_int64),
+        ("q_first_block", C.c_void_p),
+        ("kv_end_row", C.c_void_p),
     ]
 
 

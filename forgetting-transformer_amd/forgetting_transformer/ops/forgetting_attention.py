@@ -12,6 +12,7 @@ call raises.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import functools
 import math
@@ -23,7 +24,8 @@ import torch
 from . import _lib
 
 __all__ = ["forgetting_attention", "forgetting_attention_from_logits", "forgetting_attention_norm_gate",
-           "qk_norm_threshold", "ForgettingAttention", "ForgettingAttentionFromLogits", "ForgettingAttentionNormGate"]
+           "qk_norm_threshold", "record_pruning_bounds", "ForgettingAttention", "ForgettingAttentionFromLogits",
+           "ForgettingAttentionNormGate"]
 
 _DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
 
@@ -68,6 +70,27 @@ class _NoSwitch:
 
 
 _NO_SWITCH = _NoSwitch()
+
+_bound_records = None   # list that collects the pruning bounds of every call while record_pruning_bounds() is active
+
+
+@contextlib.contextmanager
+def record_pruning_bounds():
+    """Collect the pruning bounds the kernels work with, for every call made inside the ``with`` block.
+
+    The reference computes them with kernels of their own (``_find_start_index_kernel`` ``:695-745``,
+    ``_find_end_index_kernel`` ``:747-795``) whose results only ``return_start_index`` exposes, and only for the
+    forward.  Here the searches run inside the attention kernels; this context asks all three for what they found.
+    Yields a list that receives one dict per call with a threshold: ``{"fwd_first_block": (B,H,ceil(M/block_m))}``
+    from a forward, ``{"dq_first_block": (B,H,ceil(M/block_m)), "kv_end_row": (B,H,ceil(N/64))}`` from a backward
+    (int32 tensors: first key block, in blocks of ``block_n`` keys, that each query block visits, and per 64 keys the
+    query row where the dK/dV walk below them stops).  Not thread-safe; meant for tests and diagnostics."""
+    global _bound_records
+    prev, _bound_records = _bound_records, []
+    try:
+        yield _bound_records
+    finally:
+        _bound_records = prev
 
 
 def _on_device(device: torch.device):
@@ -234,10 +257,21 @@ def _fwd_workspace_bytes(B, H, M, N, D, dtype_code):
 
 
 @functools.lru_cache(maxsize=64)
+def _cached_constant_threshold(value, B, H, device):
+    t = torch.full((B, H), value, dtype=torch.float, device=device)
+    # the fill has finished before the tensor enters the cache: whichever stream reads it later needs no ordering
+    torch.cuda.current_stream(device).synchronize()
+    return t
+
+
 def _constant_threshold(value, B, H, device):
     """(B, H) fp32 tensor holding one float threshold: the same values as as_tensor + broadcast_to of the reference
-    (:104-109), filled on the device once per (value, shape, device) instead of once per call.  Read-only."""
-    return torch.full((B, H), value, dtype=torch.float, device=device)
+    (:104-109), filled on the device once per (value, shape, device) instead of once per call.  Read-only.
+    Under stream capture the tensor is filled by a kernel of the captured graph instead (a tensor created during
+    capture lives in the graph's memory pool and holds nothing until the graph runs, so it must not be cached)."""
+    if device.type != "cuda" or torch.cuda.is_current_stream_capturing():   # (CPU tensors are rejected further down)
+        return torch.full((B, H), value, dtype=torch.float, device=device)
+    return _cached_constant_threshold(value, B, H, device)
 
 
 def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale, adaptive_threshold,
@@ -344,7 +378,7 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
             y = torch.empty((B, M, H, D), dtype=q.dtype, device=device).transpose(1, 2)
             rstd = torch.empty((B, M, H), dtype=torch.float32, device=device)
         first_block = None
-        if return_start_index:
+        if return_start_index or (_bound_records is not None and adaptive_threshold is not None):
             block_m, _, _, _ = _lib.tile_config(D)
             first_block = torch.zeros((B, H, (M + block_m - 1) // block_m), dtype=torch.int32, device=device)
         args = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), log_lambda.data_ptr(), L.data_ptr(),
@@ -360,6 +394,8 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
                                    rstd.data_ptr(), eps, act)
             _lib.check(lib.fox_attn_fwd_norm_gate(C.byref(args), C.byref(epi), stream), "fox_attn_fwd_norm_gate")
 
+    if _bound_records is not None and adaptive_threshold is not None:
+        _bound_records.append({"fwd_first_block": first_block})
     saved = (q, k, v, o, L, log_lambda, seq_start, adaptive_threshold, log_fgate if gate_is_logit else None)
     if epilogue is not None:
         saved += (epilogue[0], epilogue[1], rstd)
@@ -389,9 +425,15 @@ def _backward(ctx, do):
     do = maybe_contiguous(do)
     with _on_device(device):
         stream = _stream(device)
-        # one allocation for the fp32 temporaries: rowsum(o * do) and the row sums of dS (2,B,H,M), then dlog_lambda (B,H,N)
+        # one allocation for the fp32 temporaries: rowsum(o * do) and the row sums of dS (B,H,M each), then dlog_lambda (B,H,N)
         tmp = torch.empty(2 * B * H * M + B * H * N, dtype=torch.float32, device=device)
-        delta, dlog_lambda = tmp[:2 * B * H * M], tmp[2 * B * H * M:]
+        delta, drow, dlog_lambda = tmp[:B * H * M], tmp[B * H * M:2 * B * H * M], tmp[2 * B * H * M:]
+        q_first = kv_end = None
+        if _bound_records is not None and adaptive_threshold is not None:
+            block_m, _, _, _ = _lib.tile_config(D)
+            q_first = torch.zeros((B, H, (M + block_m - 1) // block_m), dtype=torch.int32, device=device)
+            kv_end = torch.full((B, H, (N + 63) // 64), -1, dtype=torch.int32, device=device)
+            _bound_records.append({"dq_first_block": q_first, "kv_end_row": kv_end})
         dlog_fgate = None
         if gate_logit is None:
             # in the layout of the caller's log_fgate when that is a permuted dense tensor (the (B,H,T) view of
@@ -405,8 +447,10 @@ def _backward(ctx, do):
             log_lambda.data_ptr(), L.data_ptr(),
             None if seq_start is None else seq_start.data_ptr(),
             None if adaptive_threshold is None else adaptive_threshold.data_ptr(),
-            ctx.sm_scale, delta.data_ptr(), dlog_lambda.data_ptr(), None if dlog_fgate is None else dlog_fgate.data_ptr(),
-            *(dlog_fgate.stride() if dlog_fgate is not None else (0, 0, 0)))
+            ctx.sm_scale, delta.data_ptr(), drow.data_ptr(), dlog_lambda.data_ptr(),
+            None if dlog_fgate is None else dlog_fgate.data_ptr(),
+            *(dlog_fgate.stride() if dlog_fgate is not None else (0, 0, 0)),
+            None if q_first is None else q_first.data_ptr(), None if kv_end is None else kv_end.data_ptr())
         if gate_logit is None:
             _lib.check(lib.fox_attn_bwd(C.byref(args), stream), "fox_attn_bwd")
             dgate = dlog_fgate

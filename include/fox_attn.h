@@ -169,24 +169,34 @@ typedef struct fox_bwd_args {
   const int64_t* seq_start;   /* (B,) or NULL */
   const float* threshold;     /* (B,H) or NULL */
   float sm_scale;
-  float* delta;               /* (2,B,H,M) workspace, written: rowsum(o * do), then the row sums of dS */
+  float* delta;               /* (B,H,M) workspace, written by the dQ stage: rowsum(o * do) */
+  float* drow;                /* (B,H,M) workspace, written by the dQ stage, read by the dK/dV stage: row sums of dS */
   float* dlog_lambda;         /* (B,H,N) workspace, written: gradient w.r.t. c */
   float* dlog_fgate;          /* (B,H,N) written: gradient w.r.t. log_fgate */
   int64_t dlog_fgate_stride_b, dlog_fgate_stride_h, dlog_fgate_stride_n;  /* its element strides; all 0 = contiguous */
+  /* Optional outputs (NULL = not wanted): the pruning bounds the two kernels worked with, the counterparts of
+   * fox_fwd_args.first_block for the results of _find_start_index_kernel (:695-745, as the dQ kernel uses them,
+   * :1239-1261) and _find_end_index_kernel (:747-795, as the dK/dV kernel uses them, :1038-1049). */
+  int32_t* q_first_block;     /* (B,H,ceil(M/block_m)), written by fox_attn_bwd_dq: first key block (of block_n keys) each
+                                 query block visits, left padding included */
+  int32_t* kv_end_row;        /* (B,H,ceil(N/64)), written by fox_attn_bwd_dkdv: for every 64 keys, the query row at which
+                                 the walk over the query blocks below them stops (M = nothing pruned; the first row of the
+                                 walk = nothing visited).  A key tile is kv_block_n keys walked in steps of kv_block_m rows,
+                                 or, for the tiles fox_set_acp_light_limit hands to the split variant, 64 keys in steps of 64 */
 } fox_bwd_args;
 
 /*
  * The stages of the backward pass, in the order they must run on a stream:
- *   fox_attn_bwd_dq    : dq; delta = rowsum(o * do) and drow[i] = sum_j dS[i,j] into the two planes of `delta`
+ *   fox_attn_bwd_dq    : dq; delta = rowsum(o * do) and drow[i] = sum_j dS[i,j]
  *                        (_bwd_preprocess :902-943 + _find_start_index_kernel + _bwd_q_kernel :1156-1344)
- *   fox_attn_bwd_dkdv  : dk, dv, dlog_lambda[n] = drow[n-(N-M)] - sum_i dS[i,n]; reads both planes of `delta`
+ *   fox_attn_bwd_dkdv  : dk, dv, dlog_lambda[n] = drow[n-(N-M)] - sum_i dS[i,n]; reads delta and drow
  *                        (_find_end_index_kernel :747-795 + _bwd_kv_kernel :956-1143)
  *   fox_cumsum_bwd     : dlog_fgate from dlog_lambda                (:390-392)
  * fox_attn_bwd runs all three (ForgettingAttention.backward :232-400).  The reference launches the key/value
  * kernel first and lets the query kernel add its row sums into the same buffer (:1334-1344); here every stage
  * only stores, so repeating a stage (or timing it alone) leaves the result unchanged, and only the order
- * dq before dkdv matters.  fox_attn_bwd_delta writes the first plane of `delta` alone (_bwd_preprocess as a stage
- * of its own); the backward does not need it.
+ * dq before dkdv matters.  fox_attn_bwd_delta writes `delta` alone (_bwd_preprocess as a stage of its own; only
+ * dims, o, d_o and delta are read from the argument block); the backward does not need it.
  */
 int fox_attn_bwd_delta(const fox_bwd_args* args, void* stream);
 int fox_attn_bwd_dkdv(const fox_bwd_args* args, void* stream);

@@ -190,7 +190,9 @@ def forgetting_attention_ref_grads(
 
 
 def manual_backward(q, k, v, log_fgate, dout, *, seq_start=None, sm_scale=None,
-                    compute_dtype=torch.float64, out_round_dtype: Optional[torch.dtype] = None):
+                    compute_dtype=torch.float64, out_round_dtype: Optional[torch.dtype] = None,
+                    row_lo: Optional[torch.Tensor] = None, col_end: Optional[torch.Tensor] = None,
+                    kv_keep: Optional[torch.Tensor] = None):
     """The kernels' hand-derived backward, head-first tensors only.
 
     ``delta = rowsum(o * do)``            (``_bwd_preprocess`` ``:902-943``)
@@ -201,31 +203,60 @@ def manual_backward(q, k, v, log_fgate, dout, *, seq_start=None, sm_scale=None,
     ``dg = reverse inclusive cumsum(dc)``        (``:390-392``)
 
     ``out_round_dtype`` optionally rounds ``o`` the way the operator stores it
-    before ``delta`` is formed.  Returns ``(out, lse, dq, dk, dv, dc, dg)``.
+    before ``delta`` is formed.
+
+    Adaptive Computation Pruning restricts each of the three kernels to its own set of entries
+    (``:600-613``, ``:1038-1049``, ``:1239-1261``):
+
+    * ``row_lo`` ``(B, H, M)``: the forward (``out``, ``lse``) and the query-side backward (``dq`` and
+      the row sums that enter ``dc``) see, for query row ``i``, only the keys ``j >= row_lo[i]``;
+    * ``col_end`` ``(B, H, N)``: the key-side backward (``dk``, ``dv`` and the column sums that enter
+      ``dc``) sees, for key ``j``, only the query rows ``i < col_end[j]``; ``kv_keep`` ``(B, H, M, N)``
+      bool gives that set entry by entry instead.
+
+    Probabilities are ``exp(s - lse)`` with the pruned forward's ``lse`` everywhere, also for entries the
+    forward itself dropped (the key-side kernel rebuilds them from the stored ``lse``, ``:1079-1087``).
+    Returns ``(out, lse, dq, dk, dv, dc, dg)``.
     """
     B, H, M, D = q.shape
     N = k.shape[2]
     p_seq = N - M
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
+    assert col_end is None or kv_keep is None
     qf, kf, vf, dof = (x.to(compute_dtype) for x in (q, k, v, dout))
     c = cumulative_log_decay(log_fgate, seq_start, compute_dtype)
     s, valid = _scores(qf, kf, c, seq_start, sm_scale)
-    any_valid = valid.any(dim=-1, keepdim=True)
     zero = torch.zeros((), dtype=compute_dtype, device=s.device)
-    s_safe = torch.where(any_valid, s, zero)
-    lse = torch.logsumexp(s_safe, dim=-1, keepdim=True)
-    p = torch.where(valid & any_valid, torch.exp(s_safe - lse), zero)
-    out = p @ vf
+    q_keep = valid
+    if row_lo is not None:
+        j = torch.arange(N, device=q.device)
+        q_keep = valid & (j[None, None, None, :] >= row_lo[..., None])
+    any_valid = q_keep.any(dim=-1, keepdim=True)
+    s_fwd = torch.where(any_valid, s.masked_fill(~q_keep, float("-inf")), zero)
+    lse = torch.logsumexp(s_fwd, dim=-1, keepdim=True)
+    p = torch.where(valid & any_valid, torch.exp(torch.where(any_valid, s, zero) - lse), zero)
+    del s_fwd
+    out = torch.where(q_keep, p, zero) @ vf
     o_used = out if out_round_dtype is None else out.to(out_round_dtype).to(compute_dtype)
     delta = (o_used * dof).sum(-1, keepdim=True)
-    dp = dof @ vf.transpose(2, 3)
-    ds = p * (dp - delta)
+    ds = p * (dof @ vf.transpose(2, 3) - delta)
+    ds_q = torch.where(q_keep, ds, zero)
+    dq = sm_scale * (ds_q @ kf)
+    drow = ds_q.sum(dim=3)
+    del ds_q
+    if col_end is not None:
+        i = torch.arange(M, device=q.device)
+        kv_keep = i[None, None, :, None] < col_end[:, :, None, :]
+    if kv_keep is not None:
+        ds = torch.where(kv_keep, ds, zero)
+        p = torch.where(kv_keep, p, zero)
+    elif row_lo is not None:
+        raise ValueError("a pruned forward needs the key-side set as well (col_end or kv_keep)")
     dv = p.transpose(2, 3) @ dof
     dk = sm_scale * (ds.transpose(2, 3) @ qf)
-    dq = sm_scale * (ds @ kf)
     dc = -ds.sum(dim=2)
-    dc[..., p_seq:] += ds.sum(dim=3)
+    dc[..., p_seq:] += drow
     dg = torch.flip(torch.cumsum(torch.flip(dc, dims=[-1]), dim=-1), dims=[-1])
     lse_out = torch.where(any_valid[..., 0], lse[..., 0], torch.full((), float("-inf"), dtype=compute_dtype, device=s.device))
     return out, lse_out, dq, dk, dv, dc, dg

@@ -165,6 +165,59 @@ def test_manual_backward_matches_autograd(M, N, ss):
         assert mdg[..., 0].abs().max() < 1e-10
 
 
+@pytest.mark.parametrize("M,N,ss", [(40, 40, None), (24, 61, [0, 30])])
+def test_pruned_manual_backward(M, N, ss):
+    """The three entry sets of a pruned backward.  (1) When the key side keeps exactly the entries the forward
+    kept, everything is the gradient of the pruned forward: autograd through ``forgetting_attention_ref(row_lo=...)``
+    pins out, dq, dk, dv and dg.  (2) A key-side set of its own (``col_end``): dk, dv and dc from element loops that
+    rebuild every probability from the pruned forward's lse."""
+    B, H, D, sm = (2 if ss else 1), 2, 8, 0.6
+    q, k, v, g, do, seq = make_inputs(B, H, M, N, D, dtype=torch.float64, seed=21, seq_start=ss, gate_mean=0.5)
+    P = N - M
+    gen = torch.Generator().manual_seed(3)
+    # per-row lower bounds, block-shaped as the kernels' are (8 rows share a bound, a multiple of 4, never right of the row)
+    blk = torch.randint(0, N // 4 + 1, (B, H, (M + 7) // 8), generator=gen) * 4
+    row_lo = torch.minimum(blk.repeat_interleave(8, dim=-1)[..., :M], (torch.arange(M) + P) // 4 * 4)
+    qq, kk, vv, gg = (x.clone().requires_grad_() for x in (q, k, v, g))
+    out = O.forgetting_attention_ref(qq, kk, vv, gg, head_first=True, seq_start=seq, sm_scale=sm, compute_dtype=torch.float64,
+                                     row_lo=row_lo)
+    out.backward(do)
+    i, j = torch.arange(M)[:, None], torch.arange(N)[None, :]
+    kept = (j <= i + P)[None, None] & (j[None, None] >= row_lo[..., None])
+    if seq is not None:
+        kept = kept & (j[None, None] >= seq[:, None, None, None])
+    mo, ml, mdq, mdk, mdv, mdc, mdg = O.manual_backward(q, k, v, g, do, seq_start=seq, sm_scale=sm, row_lo=row_lo, kv_keep=kept)
+    for name, a, b in (("out", out, mo), ("dq", qq.grad, mdq), ("dk", kk.grad, mdk), ("dv", vv.grad, mdv), ("dg", gg.grad, mdg)):
+        assert torch.allclose(a.detach(), b, atol=1e-11, rtol=1e-9), name
+    full = O.forgetting_attention_ref(q, k, v, g, head_first=True, seq_start=seq, sm_scale=sm, compute_dtype=torch.float64)
+    assert (full - mo).abs().max() > 1e-4          # the bounds did change the result
+    # (2) key-side bound per key, block-shaped, independent of the forward's set
+    col_end = (torch.randint(0, M // 8 + 2, (B, H, (N + 3) // 4), generator=gen) * 8).clamp(max=M).repeat_interleave(4, dim=-1)[..., :N]
+    _, ml2, mdq2, mdk2, mdv2, mdc2, _ = O.manual_backward(q, k, v, g, do, seq_start=seq, sm_scale=sm, row_lo=row_lo, col_end=col_end)
+    assert torch.equal(ml, ml2) and torch.equal(mdq, mdq2)   # the query side does not see the key side's set
+    c = O.cumulative_log_decay(g, seq, torch.float64)
+    delta = (mo * do).sum(-1)
+    for b in range(B):
+        s0 = 0 if seq is None else int(seq[b])
+        for h in range(H):
+            dk_ = torch.zeros(N, D, dtype=torch.float64); dv_ = torch.zeros(N, D, dtype=torch.float64)
+            dc_ = torch.zeros(N, dtype=torch.float64)
+            for n in range(N):
+                for m in range(M):
+                    if n > m + P or n < s0 or ml[b, h, m] == float("-inf"):
+                        continue
+                    p = math.exp(float(q[b, h, m] @ k[b, h, n]) * sm + float(c[b, h, m + P] - c[b, h, n]) - float(ml[b, h, m]))
+                    ds = p * (float(do[b, h, m] @ v[b, h, n]) - float(delta[b, h, m]))
+                    if n >= row_lo[b, h, m]:
+                        dc_[m + P] += ds
+                    if m < col_end[b, h, n]:
+                        dv_[n] += p * do[b, h, m]
+                        dk_[n] += sm * ds * q[b, h, m]
+                        dc_[n] -= ds
+            assert torch.allclose(mdk2[b, h], dk_, atol=1e-10) and torch.allclose(mdv2[b, h], dv_, atol=1e-10)
+            assert torch.allclose(mdc2[b, h], dc_, atol=1e-10)
+
+
 def test_gate_gradient_closed_form():
     """dg_l = sum over (rows at or after l) x (columns before l) of dS: only score
     pairs that straddle position l contribute."""
@@ -276,6 +329,19 @@ def test_end_index_scan_is_safe(c_oracle, M, N, bm, bn, thr):
     loose = O.find_end_index_ref(c, thr, M, N, bm, bn, tight=False)
     tight_ = O.find_end_index_ref(c, thr, M, N, bm, bn, tight=True)
     assert all(t <= l for t, l in zip(tight_, loose))   # the reference's bound only ever prunes less
+    # minimality of the tight form, by brute force over every entry of every (query block x key block) rectangle
+    # (causal mask ignored, as in the scan): `end` is the end of the last query block that still holds an entry at or
+    # above the threshold, and never moves back from one key block to the next.  An off-by-one in either direction
+    # (a block too many kept, or one too many dropped) fails here.
+    floor = 0
+    for blk, end in enumerate(tight_):
+        cols = range(blk * bn, min(N, blk * bn + bn))
+        exact = floor
+        for e0 in range(0, M, bm):
+            if any(cn[P + i] - cn[j] >= np.float32(thr) for i in range(e0, min(M, e0 + bm)) for j in cols):
+                exact = max(exact, min(M, e0 + bm))
+        assert end == exact, (blk, end, exact)
+        floor = end
 
 
 def test_pruned_mass_is_bounded_by_the_auto_threshold():
