@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Forgetting Attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode|c3d64|c3d32|c3d16|shift|norm_gate|ref_sweep|acp_sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|decode|c3d64|c3d32|c3d16|shift|norm_gate|ref_sweep|acp_sweep|power]
                     [--no-extras] [--no-cpu-baseline]
 
 A step is one forward + backward pass of ``forgetting_attention`` over one batch
@@ -38,6 +38,56 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT / "forgetting-transformer_amd"))
 sys.path.insert(0, str(ROOT))
+
+
+def power_sampler(csv_path, stop_path, period_s=0.02):
+    """Child process of --workload power: polls the SMI library for socket power, shader clock, temperature and
+    throttle status until `stop_path` appears; one CSV line per sample, stamped with time.time().  Never touches HIP."""
+    import amdsmi
+    amdsmi.amdsmi_init()
+    dev = amdsmi.amdsmi_get_processor_handles()[0]
+
+    def num(x):
+        try:
+            return float(x)
+        except (TypeError, ValueError):
+            return float("nan")
+
+    with open(csv_path, "w") as f:
+        try:
+            cap = amdsmi.amdsmi_get_power_cap_info(dev)
+        except Exception as e:   # noqa: BLE001 -- the sampler reports what the library offers on this box
+            cap = {"error": repr(e)}
+        f.write("# power_cap_info " + json.dumps({k: str(v) for k, v in cap.items()}) + "\n")
+        f.write("t,socket_w,gfx_mhz,gfx_mhz_max,hotspot_c,throttle\n")
+        first = True
+        while not os.path.exists(stop_path):
+            t = time.time()
+            try:
+                m = amdsmi.amdsmi_get_gpu_metrics_info(dev)
+            except Exception as e:   # noqa: BLE001
+                f.write(f"# metrics error {e!r}\n")
+                break
+            if first:
+                f.write("# first sample keys " + json.dumps(sorted(m.keys())) + "\n")
+                first = False
+            clks = [num(c) for c in (m.get("current_gfxclks") or []) if num(c) == num(c) and 0 < num(c) < 60000]
+            w = num(m.get("current_socket_power"))
+            if not w == w or w <= 0 or w > 60000:
+                w = num(m.get("average_socket_power"))
+            mhz = sum(clks) / len(clks) if clks else num(m.get("current_gfxclk"))
+            f.write(f"{t:.4f},{w:.1f},{mhz:.1f},{max(clks) if clks else mhz:.1f},{num(m.get('temperature_hotspot')):.1f},"
+                    f"{m.get('throttle_status')}\n")
+            f.flush()
+            dt = period_s - (time.time() - t)
+            if dt > 0:
+                time.sleep(dt)
+    amdsmi.amdsmi_shut_down()
+
+
+if len(sys.argv) == 4 and sys.argv[1] == "--power-sampler":   # before torch is imported: the sampler needs none of it
+    power_sampler(sys.argv[2], sys.argv[3])
+    sys.exit(0)
 
 import torch  # noqa: E402
 
@@ -700,12 +750,117 @@ def norm_gate_report(ns):
     print(json.dumps(line))
 
 
+def power_report(ns):
+    """--workload power: socket power and shader clock beside every MFMA kernel of config 3.
+
+    A child process samples the SMI library every 20 ms while this process runs, one after the other and for at least
+    `--seconds` each: nothing (idle), the forward, the dQ kernel and the dK/dV kernel of config 3 alone, the three on
+    all-zero q, k, v, dO (same instruction stream, no data toggling), and a bf16 GEMM of the vendor library (8192^3,
+    N(0,1) data) for scale.  Per phase: average launch time, TFLOP/s of executed matmuls, and mean / max power and mean
+    clock over the samples of the phase (its first 0.5 s dropped)."""
+    import subprocess
+    import tempfile
+    from forgetting_transformer.ops import _lib
+    from forgetting_transformer.ops.forgetting_attention import _view
+
+    tmp = tempfile.mkdtemp(prefix="fox_power_")
+    csv_path, stop_path = os.path.join(tmp, "samples.csv"), os.path.join(tmp, "stop")
+    child = subprocess.Popen([sys.executable, str(Path(__file__).resolve()), "--power-sampler", csv_path, stop_path])
+    try:
+        lib = _lib.load()
+        w = WORKLOADS["c3"]
+        unit = flops_fwd(w) / 2.0
+        phases = []
+
+        def run_phase(name, fn, flops):
+            t_launch = event_time(fn, 5) if fn else 0.0
+            n = max(1, int(ns.seconds / max(t_launch, 1e-4)))
+            torch.cuda.synchronize()
+            t0 = time.time()
+            if fn is None:
+                time.sleep(ns.seconds)
+                sec = 0.0
+            else:
+                sec = event_time(fn, n, warmup=0)
+            torch.cuda.synchronize()
+            phases.append({"phase": name, "t0": t0, "t1": time.time(), "ms_per_launch": sec * 1e3, "launches": n,
+                           "tflops": flops / sec * 1e-12 if sec else 0.0})
+
+        run_phase("idle", None, 0.0)
+        for zero in (False, True):
+            tensors = synth(w, "cuda")
+            if zero:
+                tensors = tuple(torch.zeros_like(t) if i in (0, 1, 2, 4) else t for i, t in enumerate(tensors))
+            q, k, v, log_fgate, dout, _ = tensors
+            q, k, v, dout = (x.transpose(1, 2) for x in (q, k, v, dout))
+            log_fgate = log_fgate.transpose(1, 2)
+            B, H, M, D = q.shape
+            N = k.shape[2]
+            stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            dims = _lib.Dims(B, H, M, N, D, _lib.DTYPE_BF16)
+            c, lse = (torch.empty((B, H, n_), dtype=torch.float32, device="cuda") for n_ in (N, M))
+            o, dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+            delta, drow, dc, dg = (torch.empty((B, H, n_), dtype=torch.float32, device="cuda") for n_ in (M, M, N, N))
+            fwd = _lib.FwdArgs(dims, _view(q), _view(k), _view(v), _view(o), c.data_ptr(), lse.data_ptr(), None, None,
+                               1.0 / math.sqrt(D), None, None, 0)
+            bwd = _lib.BwdArgs(dims, _view(q), _view(k), _view(v), _view(o), _view(dout), _view(dq), _view(dk), _view(dv),
+                               c.data_ptr(), lse.data_ptr(), None, None, 1.0 / math.sqrt(D), delta.data_ptr(), drow.data_ptr(),
+                               dc.data_ptr(), dg.data_ptr(), 0, 0, 0, None, None)
+            _lib.check(lib.fox_cumsum_fwd(log_fgate.data_ptr(), *log_fgate.stride(), None, c.data_ptr(), B, H, N, stream), "scan")
+            tag = " (all-zero q, k, v, dO)" if zero else ""
+            run_phase("fwd" + tag, lambda: _lib.check(lib.fox_attn_fwd(C.byref(fwd), stream), "fwd"), 2 * unit)
+            run_phase("bwd_dq" + tag, lambda: _lib.check(lib.fox_attn_bwd_dq(C.byref(bwd), stream), "dq"), 3 * unit)
+            run_phase("bwd_dkdv" + tag, lambda: _lib.check(lib.fox_attn_bwd_dkdv(C.byref(bwd), stream), "dkdv"), 4 * unit)
+            del tensors, q, k, v, dout, o, dq, dk, dv
+            torch.cuda.empty_cache()
+        for zero in (False, True):
+            a = torch.zeros(8192, 8192, device="cuda", dtype=torch.bfloat16)
+            b = torch.zeros(8192, 8192, device="cuda", dtype=torch.bfloat16)
+            if not zero:
+                a.normal_()
+                b.normal_()
+            out = torch.empty_like(a)
+            run_phase("vendor GEMM 8192^3 bf16" + (" (all-zero operands)" if zero else ""),
+                      lambda: torch.matmul(a, b, out=out), 2.0 * 8192 ** 3)
+    finally:
+        open(stop_path, "w").close()
+        child.wait(timeout=30)
+    header, samples = [], []
+    for ln in open(csv_path):
+        if ln.startswith("#"):
+            header.append(ln[2:].strip())
+        elif ln[0].isdigit():
+            f = ln.strip().split(",")
+            samples.append((float(f[0]), float(f[1]), float(f[2]), float(f[3]), float(f[4]), f[5]))
+    for ph in phases:
+        sel = [x for x in samples if ph["t0"] + 0.5 <= x[0] <= ph["t1"]]
+        ph["samples"] = len(sel)
+        if sel:
+            ph["socket_w_mean"] = sum(x[1] for x in sel) / len(sel)
+            ph["socket_w_max"] = max(x[1] for x in sel)
+            ph["gfx_mhz_mean"] = sum(x[2] for x in sel) / len(sel)
+            ph["gfx_mhz_max_xcd_mean"] = sum(x[3] for x in sel) / len(sel)
+            ph["hotspot_c_max"] = max(x[4] for x in sel)
+            ph["throttle_status"] = sorted({x[5] for x in sel})
+        ph["frac_of_bf16_peak"] = ph["tflops"] / PEAK_BF16_TFLOPS
+        del ph["t0"], ph["t1"]
+    span = samples[-1][0] - samples[0][0] if len(samples) > 1 else 0.0
+    dk = next(p for p in phases if p["phase"] == "bwd_dkdv")
+    print(json.dumps({
+        "metric": "socket power and shader clock beside the MFMA kernels of config 3", "value": dk.get("socket_w_mean"),
+        "unit": "W (dK/dV kernel)", "n_gpus": 1, "higher_is_better": False, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"power: c3 kernels one at a time, {ns.seconds:g} s each, SMI sampled every 20 ms"},
+        "sampler": {"samples": len(samples), "rate_hz": len(samples) / span if span else 0.0, "notes": header},
+        "phases": phases}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift", "norm_gate", "ref_sweep", "acp_sweep"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift", "norm_gate", "ref_sweep", "acp_sweep", "power"])
+    ap.add_argument("--seconds", type=float, default=3.0, help="--workload power: duration of every phase")
     ap.add_argument("--threshold", default=None,
                     help="adaptive_threshold of the main workload: a float or 'auto' (default: no pruning); with it the "
                          "roofline entry prices the dK/dV pass against HBM, the bound of a heavily pruned step")
@@ -717,6 +872,8 @@ def main():
     if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: Forgetting Attention never communicates (every (batch, head) pair is an "
                  "independent problem), so a multi-GPU run would only replicate this measurement. Use --gpus 1.")
+    if ns.workload == "power":   # starts its sampler process before this process touches the GPU
+        return power_report(ns)
     if not torch.cuda.is_available():
         sys.exit("bench.py needs an AMD GPU (there is no CPU path for the operator)")
 
