@@ -112,12 +112,12 @@ __device__ __forceinline__ void dkdv_step(const char* q_tile, const char* do_til
 //   * the score MFMAs        S, dP   of block b+1,
 //   * the vector arithmetic  P, dS   of block b,
 //   * the accumulation MFMAs dV, dK  of block b-1,
-// which are mutually independent.  The global loads of the next tile are spread over
+// which are mutually independent (one MFMA, then a few vector instructions, four times per chunk, in source order
+// between scheduling fences).  The global loads of the next tile are spread over
 // the step as well (dma(k) issues the k-th of NDMA instructions): issued back to back
 // after the barrier by all four waves they would hold every wave's issue slot, and
 // with one wave per SIMD the matrix pipe, for over a thousand cycles per step.
-// A scheduling fence after every chunk keeps the
-// compiler from regrouping them; the LDS operands of a chunk are requested three
+// The LDS operands of a chunk are requested three
 // chunks (about twelve MFMAs) ahead, across slot boundaries, so their latency hides
 // behind the chunks in between.
 template <typename Tr, int D, int NDMA, typename Dma>
@@ -171,47 +171,49 @@ __device__ __forceinline__ void dkdv_step_interior(const char* q_tile, const cha
     // the next tile's load instructions, one every kDmaEvery chunks from the second slot on
     if constexpr (c >= NCH && (c - NCH) % kDmaEvery == 0 && (c - NCH) / kDmaEvery < NDMA)
       dma(std::integral_constant<int, (c - NCH) / kDmaEvery>{});
-    if constexpr (do_s && u < KK) {
-      s[bs] = Tr::mfma32(aq[c], kreg[u], s[bs]);
-      dp[bs] = Tr::mfma32(ado[c], vreg[u], dp[bs]);
-    }
-    if constexpr (do_c && u < 2 * DB) {
-      dvacc[u % DB] = Tr::mfma32(cdo[c], pb[bc][u / DB], dvacc[u % DB]);
-      dkacc[u % DB] = Tr::mfma32(cq[c], dsb[bc][u / DB], dkacc[u % DB]);
+    // The chunk in issue order, every group fenced so that matrix and vector instructions alternate: S MFMA, exp2 of
+    // SPC scores, dP MFMA, dS and the column sum of those scores, dV MFMA, pack P (when eight scores are complete),
+    // dK MFMA, pack dS.  S and dP accumulate in VGPRs (mfma32_vgpr_acc), so this code keeps the distance between an
+    // MFMA that writes s[b] / dp[b] and the first vector instruction that reads them (12 issued instructions).  Block
+    // b's last S MFMA opens chunk NCH-1 of slot b-1 and its first score is read in chunk 0 of slot b, after that
+    // chunk's S MFMA.  For b >= 1 the instructions in between are the 2*SPC exp2 / fma, the dP MFMA, the 2*SPC multiply
+    // / add and the 8 packs of chunk NCH-1 (it completes eight scores), then the next chunk's operand requests and
+    // S MFMA: >= 20.  dP's last MFMA is followed by 2*SPC + 8 of those, the requests, the S MFMA and 2*SPC exp2 / fma
+    // before dS reads it: >= 18.  Block 0 is computed in a slot without vector work, so its first chunk of vector
+    // work starts with explicit wait states.
+    constexpr bool mf_s = do_s && u < KK, mf_c = do_c && u < 2 * DB;
+    constexpr bool pack_due = do_v && (SPC * (u + 1)) % 8 == 0;   // eight scores complete: one MFMA operand each of P and dS
+    constexpr int hh = pack_due ? SPC * (u + 1) / 8 - 1 : 0;
+    static_assert(SPC >= 2 && NCH * SPC == 16, "the distances above count on at least two scores per chunk, eight per pack");
+    if constexpr (mf_s) Tr::mfma32_vgpr_acc(s[bs], aq[c], kreg[u]);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (do_v && bv == 0 && u == 0) {
+      asm volatile("s_nop 11");
+      __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (do_v) {
 #pragma unroll
+      for (int e = 0; e < SPC; ++e) s[bv][SPC * u + e] = __builtin_amdgcn_exp2f(fmaf(s[bv][SPC * u + e], qk_scale, -colc));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (mf_s) Tr::mfma32_vgpr_acc(dp[bs], ado[c], vreg[u]);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (do_v) {
+#pragma unroll
       for (int e = 0; e < SPC; ++e) {
-        const int r = SPC * u + e;
-        const float p = __builtin_amdgcn_exp2f(fmaf(s[bv][r], qk_scale, -colc));
-        const float ds = p * dp[bv][r];
-        s[bv][r] = p;
-        dp[bv][r] = ds;
+        const float ds = s[bv][SPC * u + e] * dp[bv][SPC * u + e];
+        dp[bv][SPC * u + e] = ds;
         csum += ds;
       }
-      if constexpr ((SPC * (u + 1)) % 8 == 0) {  // eight scores complete: pack one MFMA operand each of P and dS
-        constexpr int hh = SPC * (u + 1) / 8 - 1;
-        pb[bv][hh] = pack8<Tr>(s[bv], 8 * hh);
-        dsb[bv][hh] = pack8<Tr>(dp[bv], 8 * hh);
-      }
     }
-    constexpr int kMfmaMask = 0x008, kValuMask = 0x002, kTransMask = 0x400;
-    constexpr int n_mfma = ((do_s && u < KK) ? 2 : 0) + ((do_c && u < 2 * DB) ? 2 : 0);
-    if constexpr (do_v && n_mfma == 4) {
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(kValuMask, 2 * SPC, 0);
-        __builtin_amdgcn_sched_group_barrier(kTransMask, SPC / 2, 0);
-      }
-    } else if constexpr (do_v && n_mfma == 2) {
-#pragma unroll
-      for (int k = 0; k < 2; ++k) {
-        __builtin_amdgcn_sched_group_barrier(kMfmaMask, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(kValuMask, 4 * SPC, 0);
-        __builtin_amdgcn_sched_group_barrier(kTransMask, SPC / 2, 0);
-      }
-    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (mf_c) dvacc[u % DB] = Tr::mfma32(cdo[c], pb[bc][u / DB], dvacc[u % DB]);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (pack_due) pb[bv][hh] = pack8<Tr>(s[bv], 8 * hh);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (mf_c) dkacc[u % DB] = Tr::mfma32(cq[c], dsb[bc][u / DB], dkacc[u % DB]);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (pack_due) dsb[bv][hh] = pack8<Tr>(dp[bv], 8 * hh);
     __builtin_amdgcn_sched_barrier(0);
   });
 }
@@ -408,20 +410,26 @@ __global__ __launch_bounds__(256, (D <= 64 || DSPLIT) ? 2 : 1) void dkdv_kernel(
     if (row_lane) { rc_s0[row_slot] = rc_term(); dl_s0[row_slot] = dl_term(); }
   }
   constexpr int PER = DirectTileLoader<D, BMQ>::PER;
+  // Every tile below the first interior one is a whole tile, so the source of the loads a step spreads over its chunks
+  // is a pointer that moves back by one tile per step and an extent that is either a whole tile's or, when there is no
+  // next tile, zero (the loads then write zeros into the free buffer): no address arithmetic per step beyond that.
+  const int64_t q_back = (int64_t)BMQ * a.q.st, do_back = (int64_t)BMQ * a.d_o.st;
+  const int q_whole = qld.extent(a.q.st, 0, BMQ), do_whole = dold.extent(a.d_o.st, 0, BMQ);
+  const uint16_t *q_next = qp + (int64_t)(m_top - BMQ) * a.q.st, *do_next = dop + (int64_t)(m_top - BMQ) * a.d_o.st;
   for (int t = 0; t < n_int; t += 2) {
     wait_vmem_all();
     __syncthreads();
-    {  // tile t from buffers 0; tile t+1 (if any: otherwise an empty resource, the loads write zeros) into buffers 1
+    {  // tile t from buffers 0; tile t+1 (if any) into buffers 1
       const bool more = t + 1 < n_int;
-      const int ms = m_top - (t + 1) * BMQ;
-      if (more) issue_rows(ms);
-      const uint16_t *q_next = qp + (int64_t)ms * a.q.st, *do_next = dop + (int64_t)ms * a.d_o.st;
-      const int q_bytes = qld.extent(a.q.st, ms, more ? M : ms), do_bytes = dold.extent(a.d_o.st, ms, more ? M : ms);
+      if (more) issue_rows(m_top - (t + 1) * BMQ);
+      const int q_bytes = more ? q_whole : 0, do_bytes = more ? do_whole : 0;
       dkdv_step_interior<Tr, D, 2 * PER>(q_tile0, do_tile0, rc_s0, dl_s0, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane, [&](auto k) {
         constexpr int K = decltype(k)::value;
         if constexpr (K < PER) qld.issue_one(K, q_next, q_bytes, q_tile1);
         else dold.issue_one(K - PER, do_next, do_bytes, do_tile1);
       });
+      q_next -= q_back;
+      do_next -= do_back;
     }
     if (t + 1 >= n_int) break;
     if (row_lane) { rc_s1[row_slot] = rc_term(); dl_s1[row_slot] = dl_term(); }
@@ -429,15 +437,15 @@ __global__ __launch_bounds__(256, (D <= 64 || DSPLIT) ? 2 : 1) void dkdv_kernel(
     __syncthreads();
     {
       const bool more = t + 2 < n_int;
-      const int ms = m_top - (t + 2) * BMQ;
-      if (more) issue_rows(ms);
-      const uint16_t *q_next = qp + (int64_t)ms * a.q.st, *do_next = dop + (int64_t)ms * a.d_o.st;
-      const int q_bytes = qld.extent(a.q.st, ms, more ? M : ms), do_bytes = dold.extent(a.d_o.st, ms, more ? M : ms);
+      if (more) issue_rows(m_top - (t + 2) * BMQ);
+      const int q_bytes = more ? q_whole : 0, do_bytes = more ? do_whole : 0;
       dkdv_step_interior<Tr, D, 2 * PER>(q_tile1, do_tile1, rc_s1, dl_s1, kreg, vreg, dkacc, dvacc, csum, qk_scale, colc, lane, [&](auto k) {
         constexpr int K = decltype(k)::value;
         if constexpr (K < PER) qld.issue_one(K, q_next, q_bytes, q_tile0);
         else dold.issue_one(K - PER, do_next, do_bytes, do_tile0);
       });
+      q_next -= q_back;
+      do_next -= do_back;
       if (more && row_lane) { rc_s0[row_slot] = rc_term(); dl_s0[row_slot] = dl_term(); }
     }
   }

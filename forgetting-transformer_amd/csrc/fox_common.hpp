@@ -44,6 +44,11 @@ struct Bf16 {
   static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
+  // c += a b with the accumulator in architectural VGPRs and the B operand in accumulation registers, whatever
+  // register form the compiler picks for the kernel's other MFMAs (see mfma32_vgpr_acc below).
+  static __device__ __forceinline__ void mfma32_vgpr_acc(f32x16& c, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     bf16x2 v = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(uint32_t, v);
@@ -61,6 +66,9 @@ struct Fp16 {
   static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
+  static __device__ __forceinline__ void mfma32_vgpr_acc(f32x16& c, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     f16x2 v = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(uint32_t, v);
@@ -73,6 +81,16 @@ struct Fp16 {
   }
 };
 
+// mfma32_vgpr_acc: why an MFMA is written in assembly.  A kernel compiled for one wave per SIMD (512 registers) gets
+// every MFMA builtin in the form whose accumulator lives in the accumulation registers (AGPRs); a vector
+// instruction cannot read those, so each score that goes from an MFMA into exp2 / multiply costs a v_accvgpr_read
+// first (two per score in the dK/dV kernel, 13 % of its instruction stream, and that kernel's time follows its
+// instruction count).  The assembly form keeps such an accumulator in VGPRs and takes the loop-invariant B operand
+// (the K or V rows a wave holds) from AGPRs, where it costs nothing.  The compiler inserts the memory waits for the
+// operands of an asm statement, but not the wait states this target needs between an MFMA's write and a vector
+// instruction's read of the same registers (12 issued instructions for this 8-pass MFMA): the caller must keep
+// that distance by construction.  Back-to-back MFMAs that accumulate into the same registers need none.
+//
 // Pack eight consecutive accumulator values into one 16-byte MFMA operand.
 template <typename Tr>
 __device__ __forceinline__ u32x4 pack8(const f32x16& c, int first) {
