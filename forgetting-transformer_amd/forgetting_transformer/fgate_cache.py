@@ -121,8 +121,10 @@ class FgateDynamicCache:
             part._seen_tokens = self._seen_tokens
             for idx in range(len(self)):
                 n = self.get_seq_length(idx)
-                part._adopt(self._key_buf[idx][i:i + split_size], self._value_buf[idx][i:i + split_size],
-                            self._log_fgate_buf[idx][i:i + split_size], n)
+                # views of the filled part only: a split has no spare capacity of the parent's to write into, so its
+                # first update moves it to a buffer of its own and neither cache sees the other's later tokens
+                part._adopt(self._key_buf[idx][i:i + split_size, :, :n], self._value_buf[idx][i:i + split_size, :, :n],
+                            self._log_fgate_buf[idx][i:i + split_size, :, :n], n)
             out.append(part)
         return out
 

@@ -98,6 +98,28 @@ def test_batch_operations():
     assert cache.get_seq_length(0) == 21 and cache.get_seq_length(1) == 20
 
 
+def test_splits_and_parent_grow_independently():
+    """The reference builds a new tensor on every update (torch.cat, fgate_cache.py:107-116), so a split and its
+    parent never see each other's later tokens; the in-place cache must behave the same although a split starts
+    out as views of the parent's buffers."""
+    B, H, D = 4, 2, 8
+    cache = FgateDynamicCache(min_capacity=64)         # spare capacity in the parent's buffers
+    cache.update(*_tokens(B, H, 10, D, 0), 0)
+    before = [t.clone() for t in cache[0]]
+    parts = cache.batch_split(B, 2)
+    k1, v1, g1 = _tokens(2, H, 3, D, 5)
+    k2, v2, g2 = _tokens(B, H, 3, D, 6)
+    got_part = [t.clone() for t in parts[0].update(k1, v1, g1, 0)]     # the split grows first ...
+    got_full = [t.clone() for t in cache.update(k2, v2, g2, 0)]        # ... then the parent, over the same positions
+    for got, old, new, sl in ((got_part, before, (k1, v1, g1), slice(0, 2)), (got_full, before, (k2, v2, g2), slice(None))):
+        for x, o, n in zip(got, old, new):
+            assert torch.equal(x, torch.cat([o[sl], n], dim=2))
+    for x, o, n in zip(parts[0][0], before, (k1, v1, g1)):            # and the split still holds its own tokens
+        assert torch.equal(x, torch.cat([o[:2], n], dim=2))
+    for x, o in zip(parts[1][0], before):                              # the untouched split is unchanged
+        assert torch.equal(x, o[2:4])
+
+
 def test_shift_states_and_errors():
     cache = FgateDynamicCache()
     ks, vs = torch.zeros(2, 16), torch.ones(2, 16)

@@ -251,6 +251,34 @@ def test_single_query_matches_last_row_of_a_full_forward(fa):
         assert (start_one[:, :, 0] > 0).all() == (thr is not None)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_row_mass_in_tiny_probabilities(fa, dtype):
+    """One key outweighs every other by e^11 while the 32768 others together still hold a third of each row's mass:
+    relative to the running maximum their probabilities are 1.7e-5, below the smallest normal fp16 number.  The
+    forward's row sum adds the probabilities as rounded for the PV matrix product (a dot-product instruction against
+    ones) where the reference adds them in fp32 (tl.sum(p, 1), :650-651): if that instruction dropped subnormal
+    inputs that the matrix unit keeps, out and the log-normaliser would be off by that third.  Against the fp64 oracle."""
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    B, H, M, N, D = 1, 2, 256, 32768, 64
+    g_ = torch.Generator().manual_seed(123)
+    q = torch.randn(B, H, M, D, generator=g_) * 0.05
+    k = torch.randn(B, H, N, D, generator=g_) * 0.05
+    v = torch.randn(B, H, N, D, generator=g_)
+    q[..., 0] = 8.0
+    k[..., 0] = 0.0
+    k[:, :, 7, 0] = 11.0          # q.k / sqrt(D) = 8 * 11 / 8 = 11 for key 7, about 0 for the others
+    v[:, :, 7] = 3.0
+    gates = torch.full((B, H, N), -1e-7)
+    q, k, v = (x.to(dtype).cuda() for x in (q, k, v))
+    gates = gates.cuda()
+    out, lse, _ = ForgettingAttention.apply(q, k, v, gates, None, True, None, None, True, False)
+    ref, lse_ref = O.forgetting_attention_ref(q, k, v, gates, head_first=True, return_lse=True, compute_dtype=torch.float64)
+    share = 1.0 - torch.exp(11.0 - lse_ref).mean().item()     # mass outside the dominant key
+    assert 0.2 < share < 0.5
+    assert (lse.double() - lse_ref).abs().max().item() <= 2e-3
+    assert rel_err(out, ref) <= (REL_TOL if dtype == torch.bfloat16 else 1e-2)
+
+
 @pytest.mark.parametrize("sm_scale", [None, 0.5, 1.3])
 def test_sm_scale(fa, sm_scale):
     run_case(fa, 1, 2, 260, 260, 64, sm_scale=sm_scale, qkv_std=0.5, seed=3)
