@@ -15,7 +15,12 @@ Besides the headline value the line carries
                  stream, against the bf16 MFMA peak;
   kernels      : the same for every stage of the path;
   cpu_baseline : the PyTorch fp32 restatement of the reference's materialised-mask
-                 attention, forward only, on this host's cores, bounded to ~10 s;
+                 attention on this host's cores: forward + backward (autograd) of one
+                 (batch, head) pair of config 3, best of two runs of about 7 s each, and
+                 the forward of config 1;
+  backward_credited_frac : the five matrix products the FLOP convention credits to the
+                 backward over the time of its two kernels, against the peak (the split
+                 backward executes seven);
   acp          : pruned-tile fraction and speed-up of Adaptive Computation Pruning
                  (thresholds "auto" and -10.0) on strongly decaying gates;
   prefill      : chunked-prefill shape (M=128, N=32768, left padding), HBM GB/s;
@@ -979,6 +984,11 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    if not w["fwd_only"] and thr is None:
+        # the convention credits the backward 5 x B*H*T^2*D; its two kernels execute 3 + 4 (S and dP are recomputed in both)
+        bwd_s = stages["bwd_dq"] + stages["bwd_dkdv"]
+        line["backward_credited_frac"] = 5 * unit_flops / bwd_s * 1e-12 / PEAK_BF16_TFLOPS
+        line["backward_executed_frac"] = 7 * unit_flops / bwd_s * 1e-12 / PEAK_BF16_TFLOPS
     if not ns.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
     if not ns.no_extras and ns.workload == "c3":
