@@ -929,7 +929,7 @@ def main():
         from forgetting_transformer.ops.forgetting_attention import _view
         qh, kh = (x.detach().transpose(1, 2) if not w["head_first"] else x.detach() for x in (q, k))
         stage_thr = torch.empty((w["B"], w["H"]), dtype=torch.float32, device="cuda")
-        scratch = torch.empty((w["B"], w["H"], 2), dtype=torch.int32, device="cuda")
+        scratch = torch.empty((w["B"], w["H"], 3), dtype=torch.int32, device="cuda")
         dims = _lib.Dims(w["B"], w["H"], w["M"], w["N"], w["D"], _lib.DTYPE_BF16)
         qv, kv = _view(qh), _view(kh)
         _lib.check(_lib.load().fox_auto_threshold(C.byref(dims), C.byref(qv), C.byref(kv), 1.0 / math.sqrt(w["D"]),

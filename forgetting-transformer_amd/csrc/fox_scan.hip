@@ -3,8 +3,7 @@
 //   scan_kernel<false> : c[n]  = sum_{l<=n} g[l], with g[l] := 0 for l < seq_start
 //   scan_kernel<true>  : dg[l] = sum_{n>=l} dc[n]
 //   gate_scan_fwd/bwd  : the same two scans fused with logsigmoid of the gate logits and its derivative
-//   norm_max_kernel / threshold_kernel : the "auto" threshold from the largest row
-//                        L2 norms of q and k.
+//   norm_max_kernel    : the "auto" threshold from the largest row L2 norms of q and k.
 //
 // One workgroup scans one (batch, head) row.  Partial sums are carried in fp64 and
 // rounded once on store, so c is exactly non-increasing whenever g <= 0 (the
@@ -242,9 +241,12 @@ __global__ void zero_u32_kernel(uint32_t* p, int n) {
   if (i < n) p[i] = 0u;
 }
 
-// grid (row blocks, B*H, 2): z = 0 scans q (T = M), z = 1 scans k (T = N).
+// grid (row blocks, B*H, 2): z = 0 scans q (T = M), z = 1 scans k (T = N).  scratch holds, per (batch, head), the two
+// running maxima (float bits) and the number of workgroups that have added theirs; the workgroup that arrives last
+// turns the maxima into the threshold, so no kernel of its own is needed for that.
 template <typename Tr, int D>
-__global__ __launch_bounds__(256) void norm_max_kernel(View q, View k, int H, int M, int N, uint32_t* scratch) {
+__global__ __launch_bounds__(256) void norm_max_kernel(View q, View k, int H, int M, int N, uint32_t* scratch, float* thr,
+                                                       float sm_scale, float log_n) {
   constexpr int LPR = D / 8, RPP = 256 / LPR, ROWS = 512;
   const int tid = threadIdx.x;
   const int bh = blockIdx.y, b = bh / H, h = bh % H;
@@ -273,39 +275,45 @@ __global__ __launch_bounds__(256) void norm_max_kernel(View q, View k, int H, in
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) best = fmaxf(best, __shfl_xor(best, off));
-  if ((tid & 63) == 0) atomicMax(&scratch[bh * 2 + blockIdx.z], __float_as_uint(best));  // non-negative floats order like uints
-}
-
-template <typename Tr>
-__global__ void threshold_kernel(const uint32_t* scratch, float* thr, int n_bh, float sm_scale, float log_n) {
-  const int bh = blockIdx.x * blockDim.x + threadIdx.x;
-  if (bh >= n_bh) return;
-  const float qn = __uint_as_float(scratch[bh * 2]), kn = __uint_as_float(scratch[bh * 2 + 1]);
+  __shared__ float wave_best[4];
+  if ((tid & 63) == 0) wave_best[tid >> 6] = best;
+  __syncthreads();
+  if (tid != 0) return;
+  best = fmaxf(fmaxf(wave_best[0], wave_best[1]), fmaxf(wave_best[2], wave_best[3]));
+  uint32_t* mine = scratch + bh * 3;
+  // Non-negative floats order like uints.  The arrival is counted only after the maximum has been applied: the count's
+  // operand depends on the value the first atomic returns, and a returning atomic has been carried out where all
+  // workgroups' atomics meet.  (No fence: a device-wide release would write back the whole L2 once per workgroup.)
+  const uint32_t before = atomicMax(&mine[blockIdx.z], __float_as_uint(best));
+  uint32_t one = 1u;
+  asm volatile("" : "+v"(one) : "v"(before));
+  if (atomicAdd(&mine[2], one) != gridDim.x * 2u - 1u) return;
+  // the last workgroup of this (batch, head): every maximum has been added (read through the atomic unit as well)
+  const float qn = __uint_as_float(atomicMax(&mine[0], 0u)), kn = __uint_as_float(atomicMax(&mine[1], 0u));
   // every tensor op of the reference rounds to the input dtype
   float ub = round16<Tr>(qn * kn);
   ub = round16<Tr>(ub * sm_scale);
-  float t = round16<Tr>(2.f * ub);
-  t = round16<Tr>(t + log_n);
-  t = -t;
-  t = round16<Tr>(t - 10.f);
-  thr[bh] = t;
+  float th = round16<Tr>(2.f * ub);
+  th = round16<Tr>(th + log_n);
+  th = -th;
+  th = round16<Tr>(th - 10.f);
+  thr[bh] = th;
 }
 
 template <typename Tr>
 static hipError_t auto_threshold_t(const View& q, const View& k, int B, int H, int M, int N, int D, float sm_scale, float* thr,
                                    uint32_t* scratch, hipStream_t s) {
   const int n_bh = B * H;
-  hipLaunchKernelGGL(zero_u32_kernel, dim3((unsigned)((2 * n_bh + 255) / 256)), dim3(256), 0, s, scratch, 2 * n_bh);
+  hipLaunchKernelGGL(zero_u32_kernel, dim3((unsigned)((3 * n_bh + 255) / 256)), dim3(256), 0, s, scratch, 3 * n_bh);
   const dim3 grid((unsigned)((N + 511) / 512), (unsigned)n_bh, 2u);
+  const float log_n = (float)log((double)N);
   switch (D) {
-    case 16: hipLaunchKernelGGL((norm_max_kernel<Tr, 16>), grid, dim3(256), 0, s, q, k, H, M, N, scratch); break;
-    case 32: hipLaunchKernelGGL((norm_max_kernel<Tr, 32>), grid, dim3(256), 0, s, q, k, H, M, N, scratch); break;
-    case 64: hipLaunchKernelGGL((norm_max_kernel<Tr, 64>), grid, dim3(256), 0, s, q, k, H, M, N, scratch); break;
-    case 128: hipLaunchKernelGGL((norm_max_kernel<Tr, 128>), grid, dim3(256), 0, s, q, k, H, M, N, scratch); break;
+    case 16: hipLaunchKernelGGL((norm_max_kernel<Tr, 16>), grid, dim3(256), 0, s, q, k, H, M, N, scratch, thr, sm_scale, log_n); break;
+    case 32: hipLaunchKernelGGL((norm_max_kernel<Tr, 32>), grid, dim3(256), 0, s, q, k, H, M, N, scratch, thr, sm_scale, log_n); break;
+    case 64: hipLaunchKernelGGL((norm_max_kernel<Tr, 64>), grid, dim3(256), 0, s, q, k, H, M, N, scratch, thr, sm_scale, log_n); break;
+    case 128: hipLaunchKernelGGL((norm_max_kernel<Tr, 128>), grid, dim3(256), 0, s, q, k, H, M, N, scratch, thr, sm_scale, log_n); break;
     default: return hipErrorInvalidValue;
   }
-  hipLaunchKernelGGL((threshold_kernel<Tr>), dim3((unsigned)((n_bh + 255) / 256)), dim3(256), 0, s, scratch, thr, n_bh,
-                     sm_scale, (float)log((double)N));
   return hipGetLastError();
 }
 

@@ -345,7 +345,7 @@ def _forward(ctx, gate_is_logit, q, k, v, log_fgate, seq_start, causal, sm_scale
 
         if auto_threshold:
             adaptive_threshold = torch.empty((B, H), dtype=torch.float32, device=device)
-            scratch = torch.empty((B, H, 2), dtype=torch.int32, device=device)
+            scratch = torch.empty((B, H, 3), dtype=torch.int32, device=device)
             qv, kv = _view(q), _view(k)
             _lib.check(lib.fox_auto_threshold(C.byref(dims), C.byref(qv), C.byref(kv), sm_scale,
                                               _ptr(adaptive_threshold), _ptr(scratch), stream), "fox_auto_threshold")

@@ -109,8 +109,8 @@ int fox_gate_cumsum_bwd(const float* dc, const void* logits, int32_t logits_dtyp
 /*
  * thr[b,h] = -(2 * max_m|q| * max_n|k| * sm_scale + log N) - 10, with the row norms
  * and every intermediate rounded to the input dtype as the reference's tensor
- * arithmetic does (:95-102).  thr is (B,H) contiguous fp32; scratch is 2*B*H
- * uint32 that this call overwrites.
+ * arithmetic does (:95-102).  thr is (B,H) contiguous fp32; scratch is 3*B*H
+ * uint32 that this call overwrites (it needs no initialisation).
  */
 int fox_auto_threshold(const fox_dims* dims, const fox_view* q, const fox_view* k, float sm_scale, float* thr,
                        uint32_t* scratch, void* stream);

@@ -567,7 +567,7 @@ def test_auto_threshold_kernel(fa, dtype):
     B, H, M, N, D = 2, 3, 700, 1300, 64
     q, k, _, _, _, _ = make_inputs(B, H, M, N, D, dtype=dtype, device="cuda", seed=17)
     thr = torch.empty(B, H, device="cuda")
-    scratch = torch.empty(B, H, 2, dtype=torch.int32, device="cuda")
+    scratch = torch.empty(B, H, 3, dtype=torch.int32, device="cuda")
     dims = _lib.Dims(B, H, M, N, D, 0 if dtype == torch.bfloat16 else 1)
     qv, kv = _view(q), _view(k)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
