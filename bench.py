@@ -756,7 +756,7 @@ def norm_gate_report(ns):
 
 
 def power_report(ns):
-    """--workload power: socket power and shader clock beside every MFMA kernel of config 3.
+    """--workload power: socket power and shader clock beside every MFMA kernel of config 3 (or of `--power-of`).
 
     A child process samples the SMI library every 20 ms while this process runs, one after the other and for at least
     `--seconds` each: nothing (idle), the forward, the dQ kernel and the dK/dV kernel of config 3 alone, the three on
@@ -773,7 +773,7 @@ def power_report(ns):
     child = subprocess.Popen([sys.executable, str(Path(__file__).resolve()), "--power-sampler", csv_path, stop_path])
     try:
         lib = _lib.load()
-        w = WORKLOADS["c3"]
+        w = WORKLOADS[ns.power_of]
         unit = flops_fwd(w) / 2.0
         phases = []
 
@@ -852,9 +852,9 @@ def power_report(ns):
     span = samples[-1][0] - samples[0][0] if len(samples) > 1 else 0.0
     dk = next(p for p in phases if p["phase"] == "bwd_dkdv")
     print(json.dumps({
-        "metric": "socket power and shader clock beside the MFMA kernels of config 3", "value": dk.get("socket_w_mean"),
+        "metric": f"socket power and shader clock beside the MFMA kernels of B{w['B']} T{w['M']} H{w['H']} D{w['D']} bf16", "value": dk.get("socket_w_mean"),
         "unit": "W (dK/dV kernel)", "n_gpus": 1, "higher_is_better": False, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"power: c3 kernels one at a time, {ns.seconds:g} s each, SMI sampled every 20 ms"},
+        "config": {"workload": f"power: {ns.power_of} kernels one at a time, {ns.seconds:g} s each, SMI sampled every 20 ms"},
         "sampler": {"samples": len(samples), "rate_hz": len(samples) / span if span else 0.0, "notes": header},
         "phases": phases}))
 
@@ -866,6 +866,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["shift", "norm_gate", "ref_sweep", "acp_sweep", "power"])
     ap.add_argument("--seconds", type=float, default=3.0, help="--workload power: duration of every phase")
+    ap.add_argument("--power-of", default="c3", choices=["c3", "c3d64", "c3d32", "c3d16"],
+                    help="--workload power: the workload whose kernels run")
     ap.add_argument("--threshold", default=None,
                     help="adaptive_threshold of the main workload: a float or 'auto' (default: no pruning); with it the "
                          "roofline entry prices the dK/dV pass against HBM, the bound of a heavily pruned step")
