@@ -213,7 +213,10 @@ typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), other counters untouched
 
-template <int D, int ROWS, int NW = 4>
+// AUX is the cache-policy field of the load instruction: 0 for tiles that other workgroups read again out of L2 (the
+// usual case), kLoadNonTemporal for a stream that nobody reads twice.
+constexpr int kLoadNonTemporal = 2;
+template <int D, int ROWS, int NW = 4, int AUX = 0>
 struct DirectTileLoader {
   static constexpr int CH = D / 8;
   static constexpr int NBLK = ROWS * CH / 64;        // 1 KiB blocks per tile
@@ -247,7 +250,7 @@ struct DirectTileLoader {
     const int blk = wave + NW * j;
     if (NBLK % NW == 0 || blk < NBLK) {
       const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, bytes, 0x00020000);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(tile + blk * Tile<D>::BLOCK_BYTES), 16, voff[j], 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(tile + blk * Tile<D>::BLOCK_BYTES), 16, voff[j], 0, 0, AUX);
     }
   }
   __device__ __forceinline__ void issue(const uint16_t* base, int64_t row_stride, int row0, int row_limit, char* tile) const {

@@ -205,11 +205,11 @@ __device__ __forceinline__ void fwd_tile_pipelined(const char* k_next, const cha
 
 // The global loads of a K tile and a V tile, dealt out over the D/16 chunks of a pipelined tile:
 // dma(u) issues chunk u's share.
-template <int D>
+template <int D, int AUX>
 struct TileDma {
-  static constexpr int KK = D / 16, PER = DirectTileLoader<D, kFwdBN>::PER, PER_CHUNK = (2 * PER + KK - 1) / KK;
-  const DirectTileLoader<D, kFwdBN>& kld;
-  const DirectTileLoader<D, kFwdBN>& vld;
+  static constexpr int KK = D / 16, PER = DirectTileLoader<D, kFwdBN, 4, AUX>::PER, PER_CHUNK = (2 * PER + KK - 1) / KK;
+  const DirectTileLoader<D, kFwdBN, 4, AUX>& kld;
+  const DirectTileLoader<D, kFwdBN, 4, AUX>& vld;
   const uint16_t* k_src;
   const uint16_t* v_src;
   int k_bytes, v_bytes;
@@ -238,9 +238,14 @@ struct TileDma {
 template <int D>
 constexpr int kFwdWaves = D <= 64 ? 3 : 2;
 
-template <typename Tr, int D, bool SPLIT, bool EPI = false>
+// STREAM: the variant for shapes with a single query tile per (batch, head): every K and V tile is read by exactly one
+// workgroup, so the tile loads carry the non-temporal hint (with it the chunked-prefill shape B16 M128 N32768 H16 D128
+// takes 0.62 ms instead of 0.71).  Where tiles are shared by the workgroups of several query tiles the hint costs 16-28 %.
+template <typename Tr, int D, bool SPLIT, bool EPI = false, bool STREAM = false>
 __global__ __launch_bounds__(256, kFwdWaves<D>) void fwd_kernel(const FwdK a) {
   static_assert(!(SPLIT && EPI), "partial results of a key split are not normalised");
+  static_assert(!(STREAM && EPI), "no streaming variant with the epilogue");
+  constexpr int AUX = STREAM ? kLoadNonTemporal : 0;
   constexpr int BM = kFwdBM, BN = kFwdBN;
   constexpr int KK = D / 16, DB = (D + 31) / 32, NB = BN / 32;
   static_assert(BM == 128, "four waves of 32 rows");
@@ -284,7 +289,7 @@ __global__ __launch_bounds__(256, kFwdWaves<D>) void fwd_kernel(const FwdK a) {
   // Everything the workgroup needs first is requested before anything is waited for.  The first tile to
   // visit (the one under the end of the diagonal) does not depend on the pruning bound, so it goes
   // first; then Q, then the per-row and per-key terms; the bound search's loads queue behind them.
-  const DirectTileLoader<D, BN> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
+  const DirectTileLoader<D, BN, 4, AUX> kld(a.k.st, wave, lane), vld(a.v.st, wave, lane);
   const int n0_first = hi > 0 ? ((hi - 1) / BN) * BN : 0;
   const bool early = !SPLIT && hi > (min(seq, hi) / BN) * BN && (n0_first + BN - 1 > a0 || !(qk_scale > 0.f));
   // The tile before it is requested as well when nothing can exclude it: it still reaches the workgroup's first row
@@ -433,7 +438,7 @@ __global__ __launch_bounds__(256, kFwdWaves<D>) void fwd_kernel(const FwdK a) {
       if (more_k) issue_cn(nk);
       const uint16_t *k_src = kp + (int64_t)nk * a.k.st, *v_src = vp + (int64_t)nv * a.v.st;
       const int k_bytes = kld.extent(a.k.st, nk, more_k ? N : nk), v_bytes = vld.extent(a.v.st, nv, more_v ? N : nv);
-      const TileDma<D> dma{kld, vld, k_src, v_src, k_bytes, v_bytes, k_fill, v_fill};
+      const TileDma<D, AUX> dma{kld, vld, k_src, v_src, k_bytes, v_bytes, k_fill, v_fill};
       if (wave_has_rows) fwd_tile_pipelined<Tr, D>(k_nx, v_cur, cn_nx, qreg, oacc, m_i, l_i, qk_scale, lane, s_cur, s_nx, dma);
       else dma.all();  // a wave without query rows only moves its share of the tiles
     };
@@ -540,6 +545,9 @@ __global__ __launch_bounds__(256) void combine_kernel(const FwdK a) {
   if (d == 0) a.lse[row] = empty ? -INFINITY : mx * kLn2 + __logf(l);
 }
 
+// Query tiles per (batch, head) up to which the forward's K and V tile loads carry the non-temporal hint.
+constexpr int kStreamMaxQueryTiles = 1;
+
 // explicit instantiations: every (dtype, head dim) pair the dispatcher can reach
 #define FOX_INSTANTIATE_FWD(TR)                                          \
   template __global__ void fwd_kernel<TR, 16, false>(const FwdK);        \
@@ -554,6 +562,14 @@ __global__ __launch_bounds__(256) void combine_kernel(const FwdK a) {
   template __global__ void fwd_kernel<TR, 32, true>(const FwdK);         \
   template __global__ void fwd_kernel<TR, 64, true>(const FwdK);         \
   template __global__ void fwd_kernel<TR, 128, true>(const FwdK);        \
+  template __global__ void fwd_kernel<TR, 16, false, false, true>(const FwdK);  \
+  template __global__ void fwd_kernel<TR, 32, false, false, true>(const FwdK);  \
+  template __global__ void fwd_kernel<TR, 64, false, false, true>(const FwdK);  \
+  template __global__ void fwd_kernel<TR, 128, false, false, true>(const FwdK); \
+  template __global__ void fwd_kernel<TR, 16, true, false, true>(const FwdK);   \
+  template __global__ void fwd_kernel<TR, 32, true, false, true>(const FwdK);   \
+  template __global__ void fwd_kernel<TR, 64, true, false, true>(const FwdK);   \
+  template __global__ void fwd_kernel<TR, 128, true, false, true>(const FwdK);  \
   template __global__ void combine_kernel<TR, 16>(const FwdK);           \
   template __global__ void combine_kernel<TR, 32>(const FwdK);           \
   template __global__ void combine_kernel<TR, 64>(const FwdK);           \
@@ -564,16 +580,20 @@ FOX_INSTANTIATE_FWD(Fp16)
 template <typename Tr, int D>
 static hipError_t launch_fwd_d(const FwdK& a, int dtype, hipStream_t s) {
   if (a.epi.y.ptr && (a.M == 1 || a.splits > 1)) return hipErrorInvalidValue;  // the epilogue lives in the unsplit kernel only
+  const bool stream = a.n_mtiles <= kStreamMaxQueryTiles;  // K and V tiles that (almost) nobody reads twice
   if (a.M == 1) {  // decode step: the streaming kernel, one workgroup per (batch, head, key split)
     const hipError_t e = launch_fwd_decode(a, D, dtype, s);
     if (e != hipSuccess || a.splits <= 1) return e;
   } else if (a.splits <= 1) {
     const dim3 grid((unsigned)(a.n_mtiles * a.B * a.H));
     if (a.epi.y.ptr) hipLaunchKernelGGL((fwd_kernel<Tr, D, false, true>), grid, dim3(256), 0, s, a);
+    else if (stream) hipLaunchKernelGGL((fwd_kernel<Tr, D, false, false, true>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((fwd_kernel<Tr, D, false>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
   } else {
-    hipLaunchKernelGGL((fwd_kernel<Tr, D, true>), dim3((unsigned)(a.n_mtiles * a.splits * a.B * a.H)), dim3(256), 0, s, a);
+    const dim3 grid((unsigned)(a.n_mtiles * a.splits * a.B * a.H));
+    if (stream) hipLaunchKernelGGL((fwd_kernel<Tr, D, true, false, true>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((fwd_kernel<Tr, D, true>), grid, dim3(256), 0, s, a);
   }
   const int64_t threads = (int64_t)a.B * a.H * a.M * (D / 4);
   hipLaunchKernelGGL((combine_kernel<Tr, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, a);
