@@ -47,8 +47,8 @@ __global__ __launch_bounds__(256) void norm_gate_fwd_kernel(const NormGateK a) {
   const int h = live ? (int)(grp % a.G) : 0;
   const int64_t off = h * (int64_t)D + chunk * 8;
   float x[8], g[8], w[8], y[8];
-  unpack8v<Tr>(*reinterpret_cast<const u32x4*>(a.x + row * a.x_sr + off), x);
-  if (ACT != kActNone) unpack8v<Tr>(*reinterpret_cast<const u32x4*>(a.g + row * a.g_sr + off), g);
+  unpack8v<Tr>(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.x + row * a.x_sr + off)), x);
+  if (ACT != kActNone) unpack8v<Tr>(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.g + row * a.g_sr + off)), g);
   {
     const f32x4 w0 = *reinterpret_cast<const f32x4*>(a.w + off), w1 = *reinterpret_cast<const f32x4*>(a.w + off + 4);
 #pragma unroll
@@ -105,9 +105,9 @@ __global__ __launch_bounds__(256) void norm_gate_bwd_kernel(const NormGateK a) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int64_t r = min(rb + u, r1 - 1);
-      xv[u] = *reinterpret_cast<const u32x4*>(a.x + r * a.x_sr + off);
-      if (ACT != kActNone) gv[u] = *reinterpret_cast<const u32x4*>(a.g + r * a.g_sr + off);
-      dyv[u] = *reinterpret_cast<const u32x4*>(a.dy + r * a.dy_sr + off);
+      xv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.x + r * a.x_sr + off));
+      if (ACT != kActNone) gv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.g + r * a.g_sr + off));
+      dyv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.dy + r * a.dy_sr + off));
       rs[u] = a.rstd[r * a.G + hh];
     }
 #pragma unroll
@@ -144,8 +144,14 @@ __global__ __launch_bounds__(256) void norm_gate_bwd_kernel(const NormGateK a) {
         c1 *= 1.0f / D;
 #pragma unroll
         for (int e = 0; e < 8; ++e) dx[e] = (wdy[e] - x[e] * c1) * rs[u];
-        *reinterpret_cast<u32x4*>(a.dx + r * a.dx_sr + off) = pack8v<Tr>(dx);
-        if (ACT != kActNone) *reinterpret_cast<u32x4*>(a.dg + r * a.dg_sr + off) = pack8v<Tr>(dg);
+        // Every input is read once (non-temporal loads above).  With a gate the kernel writes two streams and the
+        // non-temporal hint on the stores pays as well (0.277 -> 0.262 ms at B4 T16384 H16 D128); with dx alone it costs.
+        if (ACT != kActNone) {
+          __builtin_nontemporal_store(pack8v<Tr>(dx), reinterpret_cast<u32x4*>(a.dx + r * a.dx_sr + off));
+          __builtin_nontemporal_store(pack8v<Tr>(dg), reinterpret_cast<u32x4*>(a.dg + r * a.dg_sr + off));
+        } else {
+          *reinterpret_cast<u32x4*>(a.dx + r * a.dx_sr + off) = pack8v<Tr>(dx);
+        }
       }
     }
   }

@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void shift_fwd_kernel(const ShiftK a) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int t = min(tb + u, t1 - 1);
-      cur[u] = *reinterpret_cast<const u32x4*>(xp + (int64_t)t * a.x_st);
+      cur[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xp + (int64_t)t * a.x_st));
       wp[u] = pw[(int64_t)t * a.w_st];
       wc[u] = cw[(int64_t)t * a.w_st];
     }
@@ -116,10 +116,10 @@ __global__ __launch_bounds__(256) void shift_bwd_kernel(const ShiftK a) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int t = max(tb - u, t0);
-      g[u] = *reinterpret_cast<const u32x4*>(gp + (int64_t)t * a.x_st);
+      g[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(gp + (int64_t)t * a.x_st));
       const u32x4 z = {0u, 0u, 0u, 0u};
       xb[u] = z;
-      if (t > 0) xb[u] = *reinterpret_cast<const u32x4*>(xp + (int64_t)(t - 1) * a.x_st);
+      if (t > 0) xb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xp + (int64_t)(t - 1) * a.x_st));
       wp[u] = pw[(int64_t)t * a.w_st];
       wc[u] = cw[(int64_t)t * a.w_st];
     }
