@@ -251,6 +251,24 @@ def test_single_query_matches_last_row_of_a_full_forward(fa):
         assert (start_one[:, :, 0] > 0).all() == (thr is not None)
 
 
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("seq,thr", [(None, None), ([0, 517], -4.0)])
+def test_single_query_tile_matches_the_last_tile_of_a_longer_call(fa, D, seq, thr):
+    """A (batch, head) with a single query tile runs through the forward's streaming instantiation (K and V tiles
+    loaded with the non-temporal hint); the same rows as the second tile of a 256-row call run through the cached one.
+    Neither call splits its keys (fewer than 16 key tiles), so both walk the same tiles in the same order: out, the
+    log-normaliser and the reported first key block are bit for bit the same."""
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    B, H, N = 2, 3, 900
+    q, k, v, g, _, _ = make_inputs(B, H, 256, N, D, device="cuda", head_first=True, seed=901 + D, gate_mean=1.0, gate_std=2.0)
+    ss = None if seq is None else torch.tensor(seq, device="cuda")
+    full, lse_full, start_full = ForgettingAttention.apply(q, k, v, g, ss, True, None, thr, True, True)
+    tail, lse_tail, start_tail = ForgettingAttention.apply(q[:, :, 128:], k, v, g, ss, True, None, thr, True, True)
+    assert torch.equal(tail, full[:, :, 128:]) and torch.equal(lse_tail, lse_full[:, :, 128:])
+    assert torch.equal(start_tail[:, :, 0], start_full[:, :, 1])
+    assert torch.isfinite(tail.float()).all() and tail.float().abs().max() > 0.1
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_row_mass_in_tiny_probabilities(fa, dtype):
     """One key outweighs every other by e^11 while the 32768 others together still hold a third of each row's mass:
