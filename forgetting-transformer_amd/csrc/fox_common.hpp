@@ -325,7 +325,9 @@ __device__ __forceinline__ void store_rows_via_lds(char* stage, const f32x16 (&a
     const int idx = idx0 + lane, row = idx / CH, ch = idx % CH;
     if ((32 * CH % kWave == 0 || idx < 32 * CH) && row0 + row < row_limit) {
       const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * RS + 16 * ch);
-      *reinterpret_cast<u32x4*>(dst + (int64_t)(row0 + row) * row_stride + 8 * ch) = v;
+      // written once, read by a later kernel at the earliest: the non-temporal hint keeps the rows from pushing K, V and
+      // Q tiles that other workgroups still want out of L2 (2-3 % of the pruned step and of small shapes, nothing at config 3)
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst + (int64_t)(row0 + row) * row_stride + 8 * ch));
     }
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -380,7 +382,7 @@ __device__ __forceinline__ void store_rows_norm_gate(char* stage, const f32x16 (
       if (act != kActNone) gv = *reinterpret_cast<const u32x4*>(gate + (int64_t)(row0 + row) * gate_stride + 8 * ch);
       const u32x4 xv = *reinterpret_cast<const u32x4*>(stage + row * RS + 16 * ch);
       const float rs = *reinterpret_cast<const float*>(stage + row * RS + 2 * D);
-      if (x_dst) *reinterpret_cast<u32x4*>(x_dst + (int64_t)(row0 + row) * x_stride + 8 * ch) = xv;
+      if (x_dst) __builtin_nontemporal_store(xv, reinterpret_cast<u32x4*>(x_dst + (int64_t)(row0 + row) * x_stride + 8 * ch));
       const f32x4 w0 = *reinterpret_cast<const f32x4*>(w + 8 * ch), w1 = *reinterpret_cast<const f32x4*>(w + 8 * ch + 4);
       u32x4 yv;
 #pragma unroll
@@ -396,7 +398,7 @@ __device__ __forceinline__ void store_rows_norm_gate(char* stage, const f32x16 (
         }
         yv[e] = Tr::pack2(y0, y1);
       }
-      *reinterpret_cast<u32x4*>(y_dst + (int64_t)(row0 + row) * y_stride + 8 * ch) = yv;
+      __builtin_nontemporal_store(yv, reinterpret_cast<u32x4*>(y_dst + (int64_t)(row0 + row) * y_stride + 8 * ch));
       if (ch == 0) rstd_dst[(int64_t)(row0 + row) * rstd_stride] = rs;
     }
   }
