@@ -326,7 +326,7 @@ __device__ __forceinline__ void store_rows_via_lds(char* stage, const f32x16 (&a
     if ((32 * CH % kWave == 0 || idx < 32 * CH) && row0 + row < row_limit) {
       const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * RS + 16 * ch);
       // written once, read by a later kernel at the earliest: the non-temporal hint keeps the rows from pushing K, V and
-      // Q tiles that other workgroups still want out of L2 (2-3 % of the pruned step and of small shapes, nothing at config 3)
+      // Q tiles that other workgroups still want out of L2 (2-3 % of a heavily pruned step and of small shapes, nothing where the kernels are matrix-bound)
       __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst + (int64_t)(row0 + row) * row_stride + 8 * ch));
     }
   }

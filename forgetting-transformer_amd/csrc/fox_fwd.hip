@@ -12,6 +12,8 @@
 // alternating buffers, so the loads of the next tile fly while the current one is
 // consumed and there is one barrier per tile.  V^T is read with the transposing
 // LDS load.
+// When a (batch, head) has a single query tile nobody reads a K or V tile twice, and the
+// loads carry the non-temporal hint (the STREAM instantiation).
 //
 // Key tiles are walked from the diagonal backwards.  Under a forget gate the
 // scores shrink with distance, so the running row maximum is set by the first
