@@ -98,7 +98,14 @@ def _on_device(device: torch.device):
     return _NO_SWITCH if torch.cuda.current_device() == device.index else torch.cuda.device(device)
 
 
+# The raw handle of the current stream without building a torch.cuda.Stream object around it (about 9 us per call
+# through the public accessor, a tenth of a small-shape step); the public accessor when this torch lacks the binding.
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device: torch.device):
+    if _raw_current_stream is not None and device.index is not None:
+        return C.c_void_p(_raw_current_stream(device.index))
     return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
