@@ -93,9 +93,12 @@ def record_pruning_bounds():
         _bound_records = prev
 
 
+_current_device = getattr(torch._C, "_cuda_getDevice", torch.cuda.current_device)   # the binding without its Python wrappers
+
+
 def _on_device(device: torch.device):
     """Context that makes ``device`` current; nothing to do (and nothing to pay) when it already is."""
-    return _NO_SWITCH if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+    return _NO_SWITCH if _current_device() == device.index else torch.cuda.device(device)
 
 
 # The raw handle of the current stream without building a torch.cuda.Stream object around it (about 9 us per call
