@@ -70,6 +70,12 @@ int check_extent(const fox_view* v, int rows, int D, const char* name) {
 // call that the variant supports.
 std::atomic<int> g_light_limit{256};   // measured crossover of the two kernels at head dim 128
 
+// Bytes of K and V together from which on a forward with one query tile per (batch, head) loads its K and V tiles
+// with the non-temporal hint (fox_set_stream_min_kv_bytes).  Such a call reads every tile once; the hint pays
+// (chunked prefill at 4 GiB: 12 %) unless the tensors are small enough to still sit in the 256 MiB last-level cache
+// when the next call on them comes (32-270 MB, called in a loop: 5-14 % faster with cached loads).
+std::atomic<int64_t> g_stream_min_kv_bytes{(int64_t)512 << 20};
+
 // The tile classes of a call: *first and *second are the classes of the launches to make (kClassAll alone,
 // kClassLight alone, or kClassLight then kClassHeavy), *limit the distance handed to the kernels.
 void tile_classes(bool pruned, bool light_ok, int* first, int* second, int* limit) {
@@ -243,6 +249,7 @@ int fwd_impl(const fox_fwd_args* args, void* workspace, int64_t workspace_bytes,
   k.sm_scale = args->sm_scale;
   k.n_mtiles = (args->dims.M + fox::kFwdBM - 1) / fox::kFwdBM;
   k.splits = 1;
+  k.stream = k.n_mtiles == 1 && (int64_t)k.B * k.H * k.N * args->dims.D * 4 >= g_stream_min_kv_bytes.load(std::memory_order_relaxed);
   if (workspace) {
     const int splits = fox::fwd_key_splits(k.B, k.H, k.M, k.N);
     const int64_t need = splits <= 1 ? 0 : (int64_t)splits * k.B * k.H * k.M * (args->dims.D + 2) * (int64_t)sizeof(float);
@@ -287,11 +294,13 @@ int fwd_impl(const fox_fwd_args* args, void* workspace, int64_t workspace_bytes,
 
 extern "C" {
 
-int fox_version(void) { return 200; }  // 0.2.0: fox_bwd_args and the scan entry points differ from 0.1.0
+int fox_version(void) { return 201; }  // 0.2.x: fox_bwd_args and the scan entry points differ from 0.1.0; 0.2.1 adds fox_set_stream_min_kv_bytes
 
 const char* fox_last_error(void) { return g_err; }
 
 int32_t fox_set_acp_light_limit(int32_t keys) { return g_light_limit.exchange(keys, std::memory_order_relaxed); }
+
+int64_t fox_set_stream_min_kv_bytes(int64_t bytes) { return g_stream_min_kv_bytes.exchange(bytes, std::memory_order_relaxed); }
 
 int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_block_n, int32_t* kv_block_m) {
   if (D != 16 && D != 32 && D != 64 && D != 128) return fail(FOX_E_ARG, "head dim must be one of 16, 32, 64, 128 (got %d)", D);

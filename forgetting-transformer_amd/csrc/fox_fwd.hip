@@ -564,7 +564,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const FwdK a) {
   if (d == 0) a.lse[row] = empty ? -INFINITY : mx * kLn2 + __logf(l);
 }
 
-// Query tiles per (batch, head) up to which the forward's K and V tile loads carry the non-temporal hint.
+// Query tiles per (batch, head) up to which the forward's K and V tile loads may carry the non-temporal hint
+// (FwdK::stream asks for it).
 constexpr int kStreamMaxQueryTiles = 1;
 
 // explicit instantiations: every (dtype, head dim) pair the dispatcher can reach
@@ -599,7 +600,7 @@ FOX_INSTANTIATE_FWD(Fp16)
 template <typename Tr, int D>
 static hipError_t launch_fwd_d(const FwdK& a, int dtype, hipStream_t s) {
   if (a.epi.y.ptr && (a.M == 1 || a.splits > 1)) return hipErrorInvalidValue;  // the epilogue lives in the unsplit kernel only
-  const bool stream = a.n_mtiles <= kStreamMaxQueryTiles;  // K and V tiles that (almost) nobody reads twice
+  const bool stream = a.stream && a.n_mtiles <= kStreamMaxQueryTiles;
   if (a.M == 1) {  // decode step: the streaming kernel, one workgroup per (batch, head, key split)
     const hipError_t e = launch_fwd_decode(a, D, dtype, s);
     if (e != hipSuccess || a.splits <= 1) return e;

@@ -35,6 +35,7 @@ struct FwdK {
   float* ws_o;     // (splits, B, H, M, D) partial accumulators
   float* ws_ml;    // (splits, B, H, M, 2) partial row maximum and row sum
   FwdEpilogue epi; // only for splits == 1 and M > 1 (the launcher rejects it otherwise)
+  bool stream;     // K and V tiles are read once and not again soon: load them with the non-temporal hint
 };
 
 struct BwdK {

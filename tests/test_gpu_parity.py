@@ -254,19 +254,51 @@ def test_single_query_matches_last_row_of_a_full_forward(fa):
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("seq,thr", [(None, None), ([0, 517], -4.0)])
 def test_single_query_tile_matches_the_last_tile_of_a_longer_call(fa, D, seq, thr):
-    """A (batch, head) with a single query tile runs through the forward's streaming instantiation (K and V tiles
-    loaded with the non-temporal hint); the same rows as the second tile of a 256-row call run through the cached one.
-    Neither call splits its keys (fewer than 16 key tiles), so both walk the same tiles in the same order: out, the
-    log-normaliser and the reported first key block are bit for bit the same."""
+    """A (batch, head) with a single query tile and enough keys runs through the forward's streaming instantiation (K and
+    V tiles loaded with the non-temporal hint; forced here for a small shape through fox_set_stream_min_kv_bytes); the
+    same rows as the second tile of a 256-row call run through the cached one.  Neither call splits its keys (fewer than
+    16 key tiles), so both walk the same tiles in the same order: out, the log-normaliser and the reported first key
+    block are bit for bit the same."""
+    from forgetting_transformer.ops import _lib
     from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    lib = _lib.load()
     B, H, N = 2, 3, 900
     q, k, v, g, _, _ = make_inputs(B, H, 256, N, D, device="cuda", head_first=True, seed=901 + D, gate_mean=1.0, gate_std=2.0)
     ss = None if seq is None else torch.tensor(seq, device="cuda")
-    full, lse_full, start_full = ForgettingAttention.apply(q, k, v, g, ss, True, None, thr, True, True)
-    tail, lse_tail, start_tail = ForgettingAttention.apply(q[:, :, 128:], k, v, g, ss, True, None, thr, True, True)
+    prev = lib.fox_set_stream_min_kv_bytes(0)
+    try:
+        full, lse_full, start_full = ForgettingAttention.apply(q, k, v, g, ss, True, None, thr, True, True)
+        tail, lse_tail, start_tail = ForgettingAttention.apply(q[:, :, 128:], k, v, g, ss, True, None, thr, True, True)
+    finally:
+        assert lib.fox_set_stream_min_kv_bytes(prev) == 0
     assert torch.equal(tail, full[:, :, 128:]) and torch.equal(lse_tail, lse_full[:, :, 128:])
     assert torch.equal(start_tail[:, :, 0], start_full[:, :, 1])
     assert torch.isfinite(tail.float()).all() and tail.float().abs().max() > 0.1
+
+
+@pytest.mark.parametrize("B,H,M,N,D", [(2, 3, 128, 900, 128), (2, 3, 100, 900, 64), (1, 2, 128, 6000, 128), (2, 2, 64, 5000, 64),
+                                        (1, 2, 77, 3000, 32), (3, 1, 128, 2100, 16)])
+@pytest.mark.parametrize("seq,thr", [(False, None), (True, -6.0)])
+def test_streaming_tile_loads_change_no_bit(fa, B, H, M, N, D, seq, thr):
+    """The same call with the streaming instantiation forced on and forced off (fox_set_stream_min_kv_bytes 0 and
+    INT64_MAX), with and without key splits, every head dim: out, log-normaliser and first key block bit for bit equal,
+    and the default limit (512 MiB) is what the setter hands back."""
+    from forgetting_transformer.ops import _lib
+    from forgetting_transformer.ops.forgetting_attention import ForgettingAttention
+    lib = _lib.load()
+    q, k, v, g, _, ss = make_inputs(B, H, M, N, D, device="cuda", head_first=True, seed=N + D, gate_mean=2.0, gate_std=1.0,
+                                    seq_start="random" if seq else None)
+    prev = lib.fox_set_stream_min_kv_bytes(0)
+    try:
+        streamed = ForgettingAttention.apply(q, k, v, g, ss, True, None, thr, True, True)
+        assert lib.fox_set_stream_min_kv_bytes(2 ** 63 - 1) == 0
+        cached = ForgettingAttention.apply(q, k, v, g, ss, True, None, thr, True, True)
+    finally:
+        lib.fox_set_stream_min_kv_bytes(prev)
+    assert prev == 512 << 20
+    for a_, b_ in zip(streamed, cached):
+        assert torch.equal(a_, b_)
+    assert streamed[0].float().abs().max() > 0.05
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -17,7 +17,7 @@ from forgetting_transformer.ops.forgetting_attention import ForgettingAttention,
 
 def test_library_exports_every_declared_symbol():
     header = (ROOT / "include" / "fox_attn.h").read_text()
-    declared = set(re.findall(r"^\s*(?:int|int32_t|const char\*)\s+(fox_\w+)\s*\(", header, flags=re.M))
+    declared = set(re.findall(r"^\s*(?:int|int32_t|int64_t|const char\*)\s+(fox_\w+)\s*\(", header, flags=re.M))
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
     lib = _lib.load()
     for name in declared:
