@@ -760,8 +760,8 @@ def power_report(ns):
 
     A child process samples the SMI library every 20 ms while this process runs, one after the other and for at least
     `--seconds` each: nothing (idle), the forward, the dQ kernel and the dK/dV kernel of config 3 alone, the three on
-    all-zero q, k, v, dO (same instruction stream, no data toggling), and a bf16 GEMM of the vendor library (8192^3,
-    N(0,1) data) for scale.  Per phase: average launch time, TFLOP/s of executed matmuls, and mean / max power and mean
+    all-zero q, k, v, dO (same instruction stream, no data toggling), a loop of register-resident MFMAs and a bf16 GEMM of
+    the vendor library (8192^3), each on N(0,1) and on all-zero operands, for scale.  Per phase: average launch time, TFLOP/s of executed matmuls, and mean / max power and mean
     clock over the samples of the phase (its first 0.5 s dropped)."""
     import subprocess
     import tempfile
@@ -818,6 +818,18 @@ def power_report(ns):
             run_phase("bwd_dkdv" + tag, lambda: _lib.check(lib.fox_attn_bwd_dkdv(C.byref(bwd), stream), "dkdv"), 4 * unit)
             del tensors, q, k, v, dout, o, dq, dk, dv
             torch.cuda.empty_cache()
+        # a loop of nothing but register-resident MFMAs (fox_probe_mfma): what the power limit leaves of the matrix peak
+        n_cu = torch.cuda.get_device_properties(0).multi_processor_count
+        sink = torch.zeros(1, device="cuda", dtype=torch.float32)
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        probe_iters = 20000
+        for zero in (False, True):
+            operands = torch.zeros(16 * 64 * 8, device="cuda", dtype=torch.bfloat16)
+            if not zero:
+                operands.normal_()
+            run_phase("MFMA loop, operands in registers" + (" (all-zero operands)" if zero else ""),
+                      lambda: _lib.check(lib.fox_probe_mfma(operands.data_ptr(), sink.data_ptr(), n_cu, probe_iters, stream), "probe"),
+                      n_cu * 4 * probe_iters * 32 * 32768.0)
         for zero in (False, True):
             a = torch.zeros(8192, 8192, device="cuda", dtype=torch.bfloat16)
             b = torch.zeros(8192, 8192, device="cuda", dtype=torch.bfloat16)

@@ -22,7 +22,7 @@ CSRC = ROOT / "csrc"
 OBJ_DIR = ROOT / "build"
 LIB_PATH = ROOT / "forgetting_transformer" / "_lib" / "libfox_attn.so"
 USAGE_PATH = LIB_PATH.with_name("kernel_resources.json")   # registers, spills, LDS of every kernel, from the compiler
-SOURCES = ["fox_fwd.hip", "fox_decode.hip", "fox_bwd.hip", "fox_scan.hip", "fox_shift.hip", "fox_norm_gate.hip", "fox_capi.hip"]
+SOURCES = ["fox_fwd.hip", "fox_decode.hip", "fox_bwd.hip", "fox_scan.hip", "fox_shift.hip", "fox_norm_gate.hip", "fox_probe.hip", "fox_capi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

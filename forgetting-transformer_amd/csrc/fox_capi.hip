@@ -294,13 +294,20 @@ int fwd_impl(const fox_fwd_args* args, void* workspace, int64_t workspace_bytes,
 
 extern "C" {
 
-int fox_version(void) { return 201; }  // 0.2.x: fox_bwd_args and the scan entry points differ from 0.1.0; 0.2.1 adds fox_set_stream_min_kv_bytes
+int fox_version(void) { return 201; }  // 0.2.x: fox_bwd_args and the scan entry points differ from 0.1.0; 0.2.1 adds fox_set_stream_min_kv_bytes and fox_probe_mfma
 
 const char* fox_last_error(void) { return g_err; }
 
 int32_t fox_set_acp_light_limit(int32_t keys) { return g_light_limit.exchange(keys, std::memory_order_relaxed); }
 
 int64_t fox_set_stream_min_kv_bytes(int64_t bytes) { return g_stream_min_kv_bytes.exchange(bytes, std::memory_order_relaxed); }
+
+int fox_probe_mfma(const void* operands, float* sink, int32_t workgroups, int32_t iters, void* stream) {
+  if (!operands || !sink) return fail(FOX_E_ARG, "fox_probe_mfma: operands and sink must not be NULL");
+  if (workgroups < 1 || workgroups > 65536 || iters < 1 || iters > (1 << 24))
+    return fail(FOX_E_ARG, "fox_probe_mfma: workgroups in [1, 65536] and iters in [1, 2^24]");
+  return check_hip(fox::launch_mfma_probe(operands, sink, workgroups, iters, (hipStream_t)stream), "fox_probe_mfma");
+}
 
 int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_block_n, int32_t* kv_block_m) {
   if (D != 16 && D != 32 && D != 64 && D != 128) return fail(FOX_E_ARG, "head dim must be one of 16, 32, 64, 128 (got %d)", D);

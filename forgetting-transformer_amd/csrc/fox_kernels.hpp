@@ -119,6 +119,7 @@ hipError_t launch_gate_cumsum_bwd(const float* dc, const void* logits, int dtype
                                   hipStream_t s);
 hipError_t launch_cumsum_bwd(const float* dc, float* dg, int64_t db, int64_t dh, int64_t dn, const int64_t* seq_start, int B, int H,
                              int N, hipStream_t s);
+hipError_t launch_mfma_probe(const void* operands, float* sink, int workgroups, int iters, hipStream_t s);  // fox_probe.hip
 hipError_t launch_auto_threshold(const View& q, const View& k, int B, int H, int M, int N, int D, int dtype, float sm_scale,
                                  float* thr, uint32_t* scratch, hipStream_t s);
 

@@ -118,6 +118,7 @@ SIGNATURES = {
     "fox_last_error": (C.c_char_p, []),
     "fox_set_acp_light_limit": (C.c_int32, [C.c_int32]),
     "fox_set_stream_min_kv_bytes": (C.c_int64, [C.c_int64]),
+    "fox_probe_mfma": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "fox_tile_config": (C.c_int, [C.c_int32] + [C.POINTER(C.c_int32)] * 4),
     "fox_cumsum_fwd": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                  C.c_int32, C.c_void_p]),

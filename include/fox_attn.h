@@ -57,6 +57,15 @@ const char* fox_last_error(void);
 int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_block_n, int32_t* kv_block_m);
 
 /*
+ * No counterpart in the reference; a measuring stick for benchmarks.  Launches `workgroups` workgroups of four
+ * waves that do nothing but 32x32x16 bf16 MFMAs on operands held in registers (32 per iteration and wave, `iters`
+ * iterations: workgroups * 4 * iters * 32 * 32768 flop).  `operands` is 16 KiB of device memory holding any 16-bit
+ * values (what the matrix pipe is fed with: on N(0,1) data the power limit of the socket, not the instruction
+ * stream, sets the rate); `sink` is one float of device memory that is never written in practice.
+ */
+int fox_probe_mfma(const void* operands, float* sink, int32_t workgroups, int32_t iters, void* stream);
+
+/*
  * Under pruning the dK/dV pass is served by two kernels: 128-key tiles whose pruning bound lies within `keys`
  * positions of their diagonal (a few query steps: a short chain of loads and stores) go to a variant that
  * splits the head dim over two waves and runs two workgroups per CU, the others to the kernel built for long

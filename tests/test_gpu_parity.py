@@ -609,6 +609,18 @@ def test_cumsum_kernels(fa):
     assert torch.equal(dg_t, dg)
 
 
+def test_mfma_probe_runs(fa):
+    """The measuring-stick loop of the power report: launches, returns, leaves its sink alone."""
+    from forgetting_transformer.ops import _lib
+    lib = _lib.load()
+    operands = torch.randn(16 * 64 * 8, device="cuda").to(torch.bfloat16)
+    sink = torch.zeros(1, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.fox_probe_mfma(operands.data_ptr(), sink.data_ptr(), 8, 50, stream), "fox_probe_mfma")
+    torch.cuda.synchronize()
+    assert sink.item() == 0.0
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_auto_threshold_kernel(fa, dtype):
     from forgetting_transformer.ops import _lib

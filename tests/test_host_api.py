@@ -117,6 +117,8 @@ def test_c_abi_rejects_bad_arguments_before_launching():
     assert lib.fox_gate_cumsum_fwd(base, 3, 1, 1, 1, None, None, base + 64, 1, 1, 8, None) == -1 and b"logits_dtype" in lib.fox_last_error()
     assert lib.fox_gate_cumsum_bwd(base, base + 64, 0, 1, 1, 1, None, base + 64, 1, 1, 1, 1, 1, 8, None) == -1 and b"alias" in lib.fox_last_error()
     assert lib.fox_gate_cumsum_bwd(base, base + 64, 0, 1, 1, 1, None, None, 1, 1, 1, 1, 1, 8, None) == -1
+    assert lib.fox_probe_mfma(None, base, 1, 1, None) == -1 and b"fox_probe_mfma" in lib.fox_last_error()
+    assert lib.fox_probe_mfma(base, base, 0, 1, None) == -1 and lib.fox_probe_mfma(base, base, 1, 0, None) == -1
     with pytest.raises(RuntimeError, match="code -1"):
         _lib.check(-1, "x")
 
