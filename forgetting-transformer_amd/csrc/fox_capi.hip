@@ -304,8 +304,8 @@ int64_t fox_set_stream_min_kv_bytes(int64_t bytes) { return g_stream_min_kv_byte
 
 int fox_probe_mfma(const void* operands, float* sink, int32_t workgroups, int32_t iters, void* stream) {
   if (!operands || !sink) return fail(FOX_E_ARG, "fox_probe_mfma: operands and sink must not be NULL");
-  if (workgroups < 1 || workgroups > 65536 || iters < 1 || iters > (1 << 24))
-    return fail(FOX_E_ARG, "fox_probe_mfma: workgroups in [1, 65536] and iters in [1, 2^24]");
+  if (workgroups < 1 || workgroups > 65536 || iters < 1 || iters > (1 << 20))   // at most about half a second per launch
+    return fail(FOX_E_ARG, "fox_probe_mfma: workgroups in [1, 65536] and iters in [1, 2^20]");
   return check_hip(fox::launch_mfma_probe(operands, sink, workgroups, iters, (hipStream_t)stream), "fox_probe_mfma");
 }
 

@@ -61,7 +61,8 @@ int fox_tile_config(int32_t D, int32_t* block_m, int32_t* block_n, int32_t* kv_b
  * waves that do nothing but 32x32x16 bf16 MFMAs on operands held in registers (32 per iteration and wave, `iters`
  * iterations: workgroups * 4 * iters * 32 * 32768 flop).  `operands` is 16 KiB of device memory holding any 16-bit
  * values (what the matrix pipe is fed with: on N(0,1) data the power limit of the socket, not the instruction
- * stream, sets the rate); `sink` is one float of device memory that is never written in practice.
+ * stream, sets the rate); `sink` is one float of device memory that is never written in practice.  workgroups in [1, 65536], iters in
+ * [1, 2^20] (about half a second per launch at most).
  */
 int fox_probe_mfma(const void* operands, float* sink, int32_t workgroups, int32_t iters, void* stream);
 
